@@ -210,6 +210,25 @@ int32_t ttbfp_gemm_bfp8b_bf16_ws(uint32_t M, uint32_t N, uint32_t K, const void 
                                  void *y_dev, uint8_t y_fmt, void *workspace_dev,
                                  uint64_t workspace_bytes, void *stream);
 
+/* ttbfp_gemm_bfp8b_bf16_ws with the scratch memory held by the library: a file-scope device array of
+ * TTBFP_STATIC_SCRATCH_BYTES that every GPU the library runs on keeps until the process ends.  For callers that
+ * cannot allocate or lend device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  The call allocates nothing (no hipMalloc / hipFree, no allocating library routine) and only launches
+ * kernels on `stream`.  Same kernels, same kernel choice and therefore the same bits as ttbfp_gemm_bfp8b_bf16_ws
+ * given a workspace of ttbfp_gemm_bfp8b_workspace_bytes(M, N, K).  A shape whose workspace would exceed
+ * TTBFP_STATIC_SCRATCH_BYTES is refused with TTBFP_RUNTIME_ERROR (8192 x 8192 x 8192 wants 128 MiB: use one of the
+ * other two entry points); a shape that uses no workspace runs exactly as ttbfp_gemm_bfp8b_bf16.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on the same GPU (two streams, two
+ * threads) race on it - serialize them.  The array keeps what the last call left; nothing in it needs clearing,
+ * each call writes every byte it later reads.  ttbfp_init resolves the array's device address (once per device);
+ * without ttbfp_init the first call on a device does.
+ * No counterpart in the reference. */
+#define TTBFP_STATIC_SCRATCH_BYTES (64ull << 20)
+uint64_t ttbfp_static_scratch_bytes(void);
+int32_t ttbfp_gemm_bfp8b_bf16_static(uint32_t M, uint32_t N, uint32_t K, const void *x_dev,
+                                     const void *w_dev, const void *bias_dev, int32_t epilogue,
+                                     void *y_dev, uint8_t y_fmt, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

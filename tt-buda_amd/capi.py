@@ -82,6 +82,10 @@ SYMBOLS = {
     "ttbfp_gemm_bfp8b_bf16_ws": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
                                                   ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
                                                   ctypes.c_uint8, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
+    "ttbfp_static_scratch_bytes": (ctypes.c_uint64, []),
+    "ttbfp_gemm_bfp8b_bf16_static": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
+                                                      ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
+                                                      ctypes.c_uint8, ctypes.c_void_p]),
 }
 
 _lib = None

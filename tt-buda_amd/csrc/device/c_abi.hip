@@ -3,6 +3,7 @@
 // thread-local text of the last failure.
 #include "../../../include/ttbfp.h"
 
+#include <atomic>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -13,9 +14,18 @@
 #include "launch.hpp"
 #include "queue_layout.hpp"
 
+// Scratch memory of ttbfp_gemm_bfp8b_bf16_static: the workspace that ttbfp_gemm_bfp8b_bf16_ws takes from its caller, held
+// by the library instead, for callers that cannot allocate.  Every device the library's code is loaded on holds its
+// own copy of the array at its own address until the process ends.  The name below is only a host-side handle of the
+// symbol: host code uses the device address that hipGetSymbolAddress returns for the current device, never the name.
+static __device__ __align__(256) unsigned char scratch[TTBFP_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_error[512] = "";
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device, nullptr until asked for
 
 int32_t fail(const char *fmt, ...)
 {
@@ -30,6 +40,22 @@ int32_t hip_status(hipError_t err, const char *what)
 {
     if (err == hipSuccess) return TTBFP_SUCCESS;
     return fail("%s: %s", what, hipGetErrorString(err));
+}
+
+// Device address of the static scratch array on `device`, which must be the calling thread's current device.  Asked
+// for once per device (ttbfp_init, or the first ttbfp_gemm_bfp8b_bf16_static on a device that was never initialised);
+// two threads that race here both get the same answer from the runtime.
+int32_t static_scratch(int device, void **out)
+{
+    if (device < 0 || device >= kMaxDevices) return fail("static scratch: device %d is beyond the %d the library keeps track of", device, kMaxDevices);
+    void *p = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!p) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail("hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
+        g_scratch_ptr[device].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return TTBFP_SUCCESS;
 }
 
 // RawUInt32 (tt::DataFormat 0xF2: integer tensors such as embedding indices, pybuda/pybuda/device_connector.py:270-277)
@@ -106,7 +132,8 @@ int32_t ttbfp_init(int32_t device)
     if (int32_t s = hip_status(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties")) return s;
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail("ttbfp_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
-    return TTBFP_SUCCESS;
+    void *p = nullptr;
+    return static_scratch(device, &p);  // set-up work (it may load the code object) done here, not in the first GEMM call
 }
 
 uint32_t ttbfp_tile_bytes(uint8_t fmt) { return ttbfp::tile_bytes(canonical(fmt)); }
@@ -425,6 +452,31 @@ int32_t ttbfp_gemm_bfp8b_bf16_ws(uint32_t M, uint32_t N, uint32_t K, const void 
     if (!panel)
         return hip_status(ttbfp::launch_gemm_bfp8b_splitk(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, (hipStream_t)stream), fn);
     return hip_status(ttbfp::launch_gemm_bfp8b_panel(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, (hipStream_t)stream), fn);
+}
+
+uint64_t ttbfp_static_scratch_bytes(void) { return TTBFP_STATIC_SCRATCH_BYTES; }
+
+int32_t ttbfp_gemm_bfp8b_bf16_static(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, const void *w_dev, const void *bias_dev,
+                                     int32_t epilogue, void *y_dev, uint8_t y_fmt, void *stream)
+{
+    const char *fn = "ttbfp_gemm_bfp8b_bf16_static";
+    bool nothing = false;
+    if (int32_t s = check_gemm(fn, M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, nothing)) return s;
+    if (nothing) return TTBFP_SUCCESS;
+    const uint64_t need = ttbfp_gemm_bfp8b_workspace_bytes(M, N, K);
+    if (need > TTBFP_STATIC_SCRATCH_BYTES)
+        return fail("%s: M=%u N=%u K=%u needs %llu bytes of scratch, the library's static scratch holds %llu; "
+                    "use ttbfp_gemm_bfp8b_bf16 (no scratch) or ttbfp_gemm_bfp8b_bf16_ws with a workspace of the caller's",
+                    fn, M, N, K, (unsigned long long)need, (unsigned long long)TTBFP_STATIC_SCRATCH_BYTES);
+    if (need == 0)  // the shape gains nothing from scratch memory: the fused kernels, which use none
+        return hip_status(ttbfp::launch_gemm_bfp8b(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, (hipStream_t)stream), fn);
+    int device = -1;
+    if (int32_t s = hip_status(hipGetDevice(&device), "hipGetDevice")) return s;
+    void *ws = nullptr;
+    if (int32_t s = static_scratch(device, &ws)) return s;
+    // Nothing in the scratch has to start at zero: the split-K planes and the panel are written in full by the first
+    // kernel before the second one reads them, so what an earlier call left there is never seen.
+    return ttbfp_gemm_bfp8b_bf16_ws(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, ws, TTBFP_STATIC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"
