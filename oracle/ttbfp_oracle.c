@@ -555,7 +555,7 @@ int oracle_prestride(const void *src, uint32_t itemsize, const uint32_t shape[4]
 
 int oracle_embedding_index(const uint32_t *index, uint32_t w, uint32_t n, uint32_t valid, uint32_t q_rt, uint32_t *out, uint32_t *cols)
 {
-    if (!q_rt || valid > n) return -1;
+    if (!q_rt) return -1;
     const uint32_t n_pad = (n + 31) / 32 * 32;
     if (n_pad % (q_rt * 32)) return -1;          /* the reference's view(w, q_rt, -1, 32) would fail */
     const uint32_t rows_per_group = n_pad / (q_rt * 32);
@@ -564,7 +564,8 @@ int oracle_embedding_index(const uint32_t *index, uint32_t w, uint32_t n, uint32
     memset(out, 0, (size_t)w * q_rt * 32 * width * 4);
     for (uint32_t iw = 0; iw < w; ++iw)
         for (uint32_t e = 0; e < n_pad; ++e) {
-            const uint32_t value = e < valid && e < n ? index[(size_t)iw * n + e] : 0xffffffffu;
+            /* zero padding first, then all-ones from position `valid` on: a vector shorter than `valid` keeps zeros in between */
+            const uint32_t value = e >= valid ? 0xffffffffu : e < n ? index[(size_t)iw * n + e] : 0u;
             const uint32_t g = e / (rows_per_group * 32), in_group = e % (rows_per_group * 32);
             const uint32_t l = in_group / 32, j = in_group % 32, a = l / 32, b = l % 32;
             out[((size_t)iw * q_rt * 32 + g * 32 + b) * width + a * 32 + j] = value;

@@ -135,8 +135,9 @@ int oracle_prestride(const void *src, uint32_t itemsize, const uint32_t shape[4]
                      uint32_t stride, void *dst, uint32_t rows_cols[2]);
 
 /* The EmbeddingIndex runtime transform (pybuda/pybuda/tensor.py:1382-1408): w index vectors of n elements, of which
- * the first `valid` are real, become the [w, 1, q_rt*32, cols] tensor the embedding queue takes.  The vector is padded
- * to a multiple of 32 with all-ones entries (also past `valid`), cut into q_rt equal groups (n padded must divide), each
+ * the first `valid` are real, become the [w, 1, q_rt*32, cols] tensor the embedding queue takes.  The vector is zero-padded
+ * to a multiple of 32 and every position from `valid` on is then set to all-ones (`valid` may exceed n: the positions in
+ * between stay zero, as in the reference's pad-then-overwrite order), cut into q_rt equal groups (n padded must divide), each
  * group written as rows of 32; with L such rows per group (padded with zero rows to L' = a multiple of 32) element j of
  * row l = 32 a + b of group g lands at out[w, 0, 32 g + b, 32 a + j].  cols = L'.  Returns 0 on success. */
 int oracle_embedding_index(const uint32_t *index, uint32_t w, uint32_t n, uint32_t valid, uint32_t q_rt, uint32_t *out,

@@ -21,7 +21,7 @@ def queue_desc(q_rt, cols_tiles):
     return q
 
 
-@pytest.mark.parametrize("n,valid,q_rt", [(32, 32, 1), (100, 100, 1), (128, 70, 1), (2048, 2048, 2), (4096, 4000, 4), (33, 33, 1)])
+@pytest.mark.parametrize("n,valid,q_rt", [(32, 32, 1), (100, 100, 1), (128, 70, 1), (2048, 2048, 2), (4096, 4000, 4), (33, 33, 1), (40, 50, 1), (40, 64, 1)])
 def test_glue_and_oracle_agree(n, valid, q_rt):
     rng = np.random.default_rng(n + valid)
     idx = rng.integers(0, 50000, (2, n), dtype=np.int32)
@@ -42,6 +42,13 @@ def test_by_hand():
     assert out[0, 0, 0].tolist() == list(range(1, 33)) and out[0, 0, 1].tolist() == list(range(33, 65))
     assert out[0, 0, 2, :6].tolist() == [65, 66, 67, 68, 69, 70] and (out[0, 0, 2, 6:] == 0xFFFFFFFF).all()
     assert not out[0, 0, 3:].any()
+    # an original shape longer than the vector (40 indices, original length 50): the reference zero-pads to 64 first and
+    # then overwrites positions 50.. with all-ones, so positions 40..49 stay zero
+    idx = np.arange(1, 41, dtype=np.uint32)
+    out = O.embedding_index(idx, 50, 1)
+    assert out[0, 0, 1, :8].tolist() == list(range(33, 41)) and not out[0, 0, 1, 8:18].any() and (out[0, 0, 1, 18:] == 0xFFFFFFFF).all()
+    got = T._embedding_index(torch.from_numpy(idx.astype(np.int32)), (50,), queue_desc(1, 1))
+    assert np.array_equal(got.numpy().view(np.uint32), out)
     # 2048 indices over two tile rows: 32 rows of 32 each; element e of the second half goes to tile row 1
     idx = np.arange(2048, dtype=np.uint32)
     out = O.embedding_index(idx, 2048, 2)

@@ -224,8 +224,9 @@ def _prestride_shape(tensor: torch.Tensor, stride_height: int, stride_width: int
 
 def _embedding_index(tensor: torch.Tensor, original_shape: Sequence[int], queue) -> torch.Tensor:
     """The EmbeddingIndex runtime transform (pybuda/pybuda/tensor.py:1382-1408): the index vector(s) of an embedding lookup
-    in the layout its RawUInt queue takes.  The vector is padded to whole rows of 32 with all-ones entries (every position
-    past the original length), dealt in order to the queue's ``q_rt`` tile rows, and each tile row's share, read as rows
+    in the layout its RawUInt queue takes.  The vector is zero-padded to whole rows of 32, every position from the original
+    length on is then set to all-ones (in that order, as the reference does: positions between the end of a vector that is
+    shorter than its original shape and that shape's length stay zero), and the result is dealt in order to the queue's ``q_rt`` tile rows, and each tile row's share, read as rows
     of 32, is laid out column-block by column-block: ``[w, 1, q_rt * 32, cols]``."""
     from ._C import DataFormat as DF
 
@@ -236,9 +237,9 @@ def _embedding_index(tensor: torch.Tensor, original_shape: Sequence[int], queue)
     w = tensor.shape[0] if tensor.dim() > 1 else 1
     n = tensor.shape[-1]
     ones = ~torch.zeros((), dtype=tensor.dtype)
-    flat = torch.full((w, n + _snap(n, 32)), int(ones), dtype=tensor.dtype)
-    valid = min(int(original_shape[-1]), n)
-    flat[:, :valid] = tensor.reshape(w, n)[:, :valid]
+    flat = torch.zeros((w, n + _snap(n, 32)), dtype=tensor.dtype)
+    flat[:, :n] = tensor.reshape(w, n)
+    flat[:, int(original_shape[-1]):] = ones
     rows = flat.shape[1] // (q_rt * 32)                      # rows of 32 per tile row of the queue
     assert rows * q_rt * 32 == flat.shape[1], "_embedding_index: the padded vector does not divide over the queue's tile rows"
     blocks = (rows + _snap(rows, 32)) // 32                  # column blocks of 32 rows each
