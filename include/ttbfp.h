@@ -59,6 +59,10 @@ extern "C" {
 #define TTBFP_EPILOGUE_NONE 0
 #define TTBFP_EPILOGUE_GELU 1
 #define TTBFP_EPILOGUE_GELU_TANH 2
+/* ORed into the epilogue argument: bias_dev holds N fp32 values instead of N bf16 ones.  For the sum over a stack of z
+ * weights (the matmul's accumulate attribute, pybuda/pybuda/op/eval/buda/matmul.py:236,306-307), whose bias term z * bias
+ * is not a bf16 value in general. */
+#define TTBFP_EPILOGUE_BIAS_F32 0x100
 
 /* Text of the last failure on this thread ("" if none). The pointer stays valid until the next
  * failing call on the same thread. */
@@ -97,6 +101,9 @@ int32_t ttbfp_memcpy_d2d(void *dst_dev, const void *src_dev, uint64_t bytes, voi
 int32_t ttbfp_pointer_is_device(const void *ptr);
 int32_t ttbfp_stream_create(void **out_stream);
 int32_t ttbfp_stream_destroy(void *stream);
+/* Waits for all work queued on the current device, on any stream.  The host layer calls it before it reads a tensor that
+ * already lives in device memory: the stream that produced it is not known at this boundary. */
+int32_t ttbfp_device_synchronize(void);
 /* Waits at most timeout_s seconds (<= 0: forever); TTBFP_TIMEOUT_ERROR when the work has not
  * finished by then - the status get_output / push_input return on a timeout (backend.py:346-371). */
 int32_t ttbfp_stream_synchronize(void *stream, int32_t timeout_s);
@@ -107,7 +114,8 @@ int32_t ttbfp_stream_synchronize(void *stream, int32_t timeout_s);
  * tt_PytorchTensorDesc, backend_api.cpp:489-560) -> tiles of faces in dst_fmt.  This is the
  * conversion inside tt::backend::tilize_tensor and push_input (backend_api.cpp:688-693, 704).
  * dst_bytes must be at least ttbfp_packed_size(dst_fmt, shape).  Legal pairs: src in
- * {Float32, Float16_b}; dst in {Bfp8_b, Bfp4_b, Bfp2_b, Float32 (fp32 source only), Float16_b};
+ * {Float32, Float16_b}; dst in {Bfp8_b, Bfp4_b, Bfp2_b, Float32, Float16_b} (a Float16_b source widens exactly into
+ * Float32 tiles through the general kernel: the host layer's full-precision mode, not a conversion of the hot path);
  * a Float16 source goes with dst in {Bfp8, Bfp4, Bfp2, Float16} and with nothing else
  * (pybuda/pybuda/device_connector.py:177-201); RawUInt32 goes to RawUInt32 tiles, a pure permutation
  * of 32-bit elements (the queues of embedding indices: device_connector.py:203-225, 270-277). */
@@ -164,6 +172,25 @@ int32_t ttbfp_unpack_untilize_queue(const void *src_dev, uint8_t src_fmt, const 
                                     uint8_t dst_fmt, const uint64_t dst_strides_bytes[4], void *dst_dev,
                                     void *stream);
 
+/* The two conversions for a tensor whose rows and columns are not multiples of 32, with the padding and the narrowing
+ * that pybuda does on the host around the boundary (pad_pytorch_tensor_to_buda / narrow_buda_tensor_to_pytorch,
+ * pybuda/pybuda/tensor.py:805-954; pad_to_buda_shape, pybuda/csrc/tt_torch_device/tt_device.cpp:153-189) done inside the
+ * launch instead.  `shape` is the shape of the row-major memory, rows and columns >= 1; the tiles cover it rounded up to
+ * multiples of 32 (align_up_tile, tt_device.hpp:205-210).
+ *  - ttbfp_tilize_pack_padded: elements past the memory's rows / columns pack as zeros ("constant" mode), or, with
+ *    replicate_rows / replicate_cols = 1, as copies of the single row / column ("replicate", legal only for a dimension
+ *    of size 1: the tile-broadcast dims of tensor.py:848-856).  layout NULL: header-less tiles in one run as
+ *    ttbfp_tilize_pack writes them (buffer_pitch_bytes ignored), else the buffers of a queue as ttbfp_tilize_pack_queue.
+ *  - ttbfp_unpack_untilize_narrow: only the shape[2] x shape[3] corner of every slice is written to dst.
+ * A shape that is tile aligned gives exactly the unpadded calls. */
+int32_t ttbfp_tilize_pack_padded(const void *src_dev, uint8_t src_fmt, const uint32_t shape[4],
+                                 const uint64_t strides_bytes[4], uint32_t replicate_rows, uint32_t replicate_cols,
+                                 uint8_t dst_fmt, int32_t rounding, const ttbfp_queue_layout *layout,
+                                 uint64_t buffer_pitch_bytes, void *dst_dev, uint64_t dst_bytes, void *stream);
+int32_t ttbfp_unpack_untilize_narrow(const void *src_dev, uint8_t src_fmt, const uint32_t shape[4],
+                                     const ttbfp_queue_layout *layout, uint64_t buffer_pitch_bytes, uint8_t dst_fmt,
+                                     const uint64_t dst_strides_bytes[4], void *dst_dev, void *stream);
+
 /* The prestriding transform that push_input applies when the queue descriptor carries a tt::Stride
  * (backend_api.cpp:392-407; set for the activation of a strided convolution by
  * pybuda/pybuda/ttdevice.py:1437-1444 with xy_offsets = [(x, y) for y in range(s) for x in range(s)]).
@@ -184,7 +211,7 @@ int32_t ttbfp_prestride(const void *src_dev, uint32_t itemsize, const uint32_t s
  * pybuda/csrc/passes/amp.cpp:474-484).
  *   x_dev     bf16 row-major, contiguous, M x K
  *   w_dev     W packed as by ttbfp_tilize_pack of the row-major [1,1,K,N] tensor to Bfp8_b
- *   bias_dev  bf16 [N] or NULL (the row the reference broadcasts: matmul.py:247-249)
+ *   bias_dev  bf16 [N] (fp32 [N] with TTBFP_EPILOGUE_BIAS_F32) or NULL (the row the reference broadcasts: matmul.py:247-249)
  *   y_dev     row-major, contiguous, M x N in y_fmt (Float16_b: round to nearest even; Float32)
  * M, N and K must be multiples of 32. */
 int32_t ttbfp_gemm_bfp8b_bf16(uint32_t M, uint32_t N, uint32_t K, const void *x_dev,
@@ -209,6 +236,13 @@ int32_t ttbfp_gemm_bfp8b_bf16_ws(uint32_t M, uint32_t N, uint32_t K, const void 
                                  const void *w_dev, const void *bias_dev, int32_t epilogue,
                                  void *y_dev, uint8_t y_fmt, void *workspace_dev,
                                  uint64_t workspace_bytes, void *stream);
+
+/* Y[M,N] = epilogue(X[M,K] * W[K,N] + bias[N]), all fp32, row-major, contiguous, any M, N, K > 0; epilogue without
+ * TTBFP_EPILOGUE_BIAS_F32 (the bias is always fp32).  The golden matmul (pybuda/pybuda/op/eval/buda/matmul.py:233-249) on
+ * unquantized operands: what the backend evaluates when its configuration says ignore_data_format_precision
+ * (pybuda/csrc/backend_api/backend_api.cpp:261-275).  Plain fp32 FMAs; a verification path, not a fast one. */
+int32_t ttbfp_gemm_f32(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, const void *w_dev,
+                       const void *bias_dev, int32_t epilogue, void *y_dev, void *stream);
 
 /* ttbfp_gemm_bfp8b_bf16_ws with the scratch memory held by the library: a file-scope device array of
  * TTBFP_STATIC_SCRATCH_BYTES that every GPU the library runs on keeps until the process ends.  For callers that

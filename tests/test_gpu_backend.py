@@ -379,9 +379,9 @@ def test_op_module_weight_stack_and_accumulate(bias_scale):
     wd = w.dequantize().cpu()
     if bias_scale is None:
         bias = None
-    elif bias_scale == 0.02:  # multiples of 1/64 up to 8/64: Z times the bias is a bf16 value, so it rides in the GEMM
+    elif bias_scale == 0.02:  # multiples of 1/64 up to 8/64: Z times the bias is a bf16 value
         bias = (torch.randint(-8, 9, (1, 1, 32, N)).float() / 64).bfloat16()
-    else:  # Z times the bias needs more than eight significant bits: added after the GEMM in fp32
+    else:  # Z times the bias needs more than eight significant bits: it rides in the GEMM's epilogue as an fp32 bias
         bias = (torch.randn(1, 1, 32, N) * bias_scale).bfloat16()
         assert not torch.equal((bias.float() * Z).bfloat16().float(), bias.float() * Z)
     golden = torch.matmul(x.float(), wd)

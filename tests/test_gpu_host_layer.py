@@ -1,0 +1,358 @@
+"""GPU tests of the host layer's behaviour around the conversions: the golden-precision switch, tensor entries of a saved
+device image, padding and narrowing at the boundary, device-resident sources, overlap of pushers and readers on one
+queue, and the block pools."""
+import json
+import os
+import sys
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from tt_buda_amd import tensor as T
+from tt_buda_amd import tti
+from tt_buda_amd._C import DataFormat as DF
+from tt_buda_amd._C import backend_api as B
+from tt_buda_amd.backend import BackendAPI
+
+pytestmark = pytest.mark.gpu
+OK, ERR, TIMEOUT = B.BackendStatusCode.Success, B.BackendStatusCode.RuntimeError, B.BackendStatusCode.TimeoutError
+RAM = B.IOType.RandomAccess
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def api():
+    a = BackendAPI(0)
+    yield a
+    a.shutdown()
+
+
+def bf16_bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16).reshape(-1)
+
+
+def read(q, fp32=False, pop=True, **kw):
+    out = B.PytorchTensorDesc()
+    if fp32:
+        out.format = DF.Float32
+    assert B.get_output(q, out, True, 1, -1, **kw) == OK, B.last_error()
+    t = T.tensor_desc_to_pytorch_tensor(out).clone()
+    assert B.free_tensor(out) == OK
+    if pop:
+        assert B.pop_output(q, True, 1) == OK
+    return t
+
+
+# ------------------------------------------------------------------------------------------------
+# golden precision switch (pybuda/csrc/backend_api/backend_api.cpp:243-281, pybuda/pybuda/verify/config.py:67,166-167)
+# ------------------------------------------------------------------------------------------------
+
+def matmul_program(api, tag, x, w, b, gelu):
+    M, K, N = x.shape[2], x.shape[3], w.shape[3]
+    qx = api.create_queue(tag + "_x", DF.Float16_b, (1, M, K))
+    qw = api.create_queue(tag + "_w", DF.Bfp8_b, (1, K, N), 1, RAM)
+    qb = api.create_queue(tag + "_b", DF.Float16_b, (1, 32, N), 1, RAM)
+    qy = api.create_queue(tag + "_y", DF.Float16_b, (1, M, N))
+    api.push_input(qw, T.pytorch_tensor_to_tensor_desc(w), True, 1, 0)
+    api.push_input(qb, T.pytorch_tensor_to_tensor_desc(b), True, 1, 0, True, False)  # one row, broadcast to its tile
+    api.push_to_queues([qx], [x], single_input=True)
+    assert api.be_api.run_matmul(tag + "_x", tag + "_w", tag + "_b", tag + "_y", gelu=gelu) == OK, B.last_error()
+    return qy
+
+
+def test_golden_precision_switch():
+    """The same program on two backends: with ignore_data_format_precision the queues keep fp32 tiles whatever their
+    declared formats and the matmul is an fp32 matmul of the tensors as pushed; without it every queue quantizes to its
+    format and the matmul runs on the dequantized values.  Each is held to its own statement, and the difference of the
+    two results is the effect of the quantization: the weight error propagated through the product, plus the rounding
+    of the result queue."""
+    say("golden precision switch")
+    M, K, N = 128, 256, 192
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(1, 1, M, K, generator=g)          # fp32 activations: Float16_b queue -> truncated to bf16 when quantizing
+    w = torch.randn(1, 1, K, N, generator=g) * 0.05
+    b = torch.randn(1, 1, 1, N, generator=g) * 0.05
+
+    quant = BackendAPI(0)                              # a device backend honours the formats by default
+    full = BackendAPI(0, golden_ignore_df_precision=True)
+    try:
+        assert not quant.be_api.get_config().ignore_data_format_precision and full.be_api.get_config().ignore_data_format_precision
+        yq = read(matmul_program(quant, "q", x, w, b, gelu=True), fp32=True)[0, 0]
+        qy_full = matmul_program(full, "f", x, w, b, gelu=True)
+        assert full.be_api.queue_storage_format("f_w") == DF.Float32 and full.be_api.queue_storage_format("f_y") == DF.Float32
+        assert quant.be_api.queue_storage_format("q_w") == DF.Bfp8_b
+        assert qy_full.data_format == DF.Float16_b  # the declared format is still what the descriptor says
+        yf = read(qy_full)[0, 0]
+        assert yf.dtype == torch.float32
+    finally:
+        quant.shutdown()
+        full.shutdown()
+
+    exact = torch.nn.functional.gelu(x[0, 0].double() @ w[0, 0].double() + b[0, 0, 0].double())
+    assert float((yf.double() - exact).norm() / exact.norm()) < 2e-6  # fp32 evaluation of the unquantized tensors
+
+    xq = torch.from_numpy(O.unpack_untilize(O.tilize_pack(x.numpy(), O.Float16_b), O.Float16_b, (1, 1, M, K), O.Float32))[0, 0]
+    wq = torch.from_numpy(O.dequant_weight(O.tilize_pack(w.numpy(), O.Bfp8_b), K, N))
+    bq = torch.from_numpy(O.unpack_untilize(O.tilize_pack(T.pad_pytorch_tensor_to_buda(b, [-2]).numpy(), O.Float16_b), O.Float16_b,
+                                            (1, 1, 32, N), O.Float32))[0, 0, 0]
+    quantized = torch.nn.functional.gelu(xq.double() @ wq.double() + bq.double())
+    assert float((yq.double() - quantized.bfloat16().double()).norm() / quantized.norm()) < 1e-3
+    # the two settings differ by the quantization error and by nothing else
+    diff, want_diff = (yf.double() - yq.double()), (exact - quantized.bfloat16().double())
+    assert float(diff.norm() / exact.norm()) > 1e-3          # the switch does something
+    # (to within the few results whose fp32 and float64 evaluations round to different bf16 neighbours)
+    assert float((diff - want_diff).norm() / want_diff.norm()) < 5e-2
+
+
+def test_full_precision_queues_keep_tensors_bit_for_bit():
+    say("full precision round trip")
+    api = BackendAPI(0, golden_ignore_df_precision=True)
+    try:
+        g = torch.Generator().manual_seed(32)
+        x = torch.randn(1, 2, 64, 96, generator=g) * 3
+        for fmt, src in ((DF.Bfp4_b, x), (DF.Bfp2_b, x.bfloat16()), (DF.Float16_b, x)):
+            q = api.create_queue(f"keep_{fmt}", fmt, (2, 64, 96))
+            api.push_to_queues([q], [src], single_input=True)
+            back = read(q)
+            assert back.dtype == torch.float32 and torch.equal(back, src.float())
+        qa = api.create_queue("keep_half", DF.Bfp8, (2, 64, 96))
+        assert api.be_api.queue_storage_format("keep_half") == DF.Float16
+        api.push_to_queues([qa], [x.half()], single_input=True)
+        assert torch.equal(read(qa), x.half())
+        # a pre-tilized tensor must be in the format the queue holds; tilize_tensor with the queue's own descriptor is
+        qt = api.create_queue("keep_tbin", DF.Bfp8_b, (2, 64, 96), 1, RAM)
+        tilized = B.tilize_tensor(qt, T.pytorch_tensor_to_tensor_desc(x))
+        assert tilized.format == DF.Float32 and tilized.buf_size_bytes == 2 * 64 * 96 * 4
+        assert B.push_input(qt, tilized, 1, 0) == OK
+        B.free_tensor(tilized)
+        assert torch.equal(read(qt, pop=False), x)
+        foreign = B.DramIODesc()
+        foreign.bufq_target_format = DF.Bfp8_b
+        packed = B.tilize_tensor(foreign, T.pytorch_tensor_to_tensor_desc(x))
+        assert packed.format == DF.Bfp8_b and B.push_input(qt, packed, 1, 0) == ERR and "differs from the format the queue holds" in B.last_error()
+        B.free_tensor(packed)
+    finally:
+        api.shutdown()
+
+
+def test_backend_config_mirrors_the_reference_surface():
+    cfg = B.BackendConfig(B.BackendType.Hip, B.BackendDevice.MI355X, B.DeviceMode.CompileAndRun, 2, "out", "", "")
+    assert (cfg.optimization_level, cfg.output_dir, cfg.ignore_data_format_precision) == (2, "out", False)
+    cfg.set_golden_ignore_df_precision(True)
+    cfg.set_performance_trace_args("--perf-level 1")
+    cfg.set_runtime_args("--foo")
+    assert cfg.ignore_data_format_precision and cfg.perf_desc_args == "--perf-level 1" and cfg.runtime_args == "--foo"
+    os.environ["TT_BACKEND_GOLDEN_QUANTIZE"] = "1"
+    try:
+        forced = BackendAPI(0, golden_ignore_df_precision=True)  # the environment wins, as in pybuda/pybuda/verify/config.py:166-167
+        assert not forced.be_api.get_config().ignore_data_format_precision
+        forced.shutdown()
+    finally:
+        del os.environ["TT_BACKEND_GOLDEN_QUANTIZE"]
+
+
+# ------------------------------------------------------------------------------------------------
+# tensor entries of a saved device image (pybuda/pybuda/tti/archive.py:52-147)
+# ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dump", [tti.TTIDumpFormat.BACKEND_TILIZED, tti.TTIDumpFormat.BACKEND, tti.TTIDumpFormat.DEFAULT])
+def test_tti_tensor_entries_round_trip(api, tmp_path, dump):
+    """tilize_tensor -> binarize -> JSON entry -> load_tensor_from_disk -> push_input -> get_output, for a Bfp8_b weight on a
+    2 x 2 grid of buffers and a Bfp4_b one in plain order; the entries carry the reference's keys."""
+    say("tti", dump)
+    g = torch.Generator().manual_seed(41)
+    params = {"layer.0.weight": torch.randn(1, 1, 128, 192, generator=g) * 0.02, "nested": {"layer.1/weight": torch.randn(1, 1, 64, 64, generator=g)}}
+    tag = dump.name.lower()
+    api.create_queue("layer.0.weight", DF.Bfp8_b, (1, 128, 192), 1, RAM, grid=(2, 2), ublock=(1, 3))
+    api.create_queue("layer.1/weight", DF.Bfp4_b, (1, 64, 64), 1, RAM)
+    directory = str(tmp_path / tag)
+    try:
+        path = tti.save_tensors(params, directory, dump, api)
+        doc = json.load(open(path))
+        assert doc["tti_dump_format"] == dump.name and doc["tti_version"] == "1.1.0"
+        e0, e1 = doc["tensors"]["layer.0.weight"], doc["tensors"]["nested"]["layer.1/weight"]
+        if dump == tti.TTIDumpFormat.DEFAULT:
+            assert e0 == os.path.join("tensors", "torch.Tensor.layer.0.weight.pkl") and e1.endswith("torch.Tensor.layer.1_weight.pkl")
+            loaded = tti.load_tensors(directory)
+            assert torch.equal(loaded["layer.0.weight"], params["layer.0.weight"])
+            return
+        assert e0["bin"] == os.path.join("tensors", "torch.Tensor.layer.0.weight." + dump.extension())
+        assert (e0["itemsize"], e0["shape"], e0["strides"], e0["dim"]) == (4, [1, 1, 128, 192], [98304, 98304, 768, 4], 4)
+        if dump == tti.TTIDumpFormat.BACKEND_TILIZED:
+            assert (e0["format"], e0["num_buffers"], e0["buf_size_bytes"]) == ("Bfp8_b", 4, 6 * 1088)
+            assert (e1["format"], e1["num_buffers"], e1["buf_size_bytes"]) == ("Bfp4_b", 1, 4 * 576)
+            assert os.path.getsize(os.path.join(directory, e0["bin"])) == 24 * 1088
+        else:
+            assert e0["format"] == "Float32" and "num_buffers" not in e0
+            assert os.path.getsize(os.path.join(directory, e0["bin"])) == 128 * 192 * 4
+        loaded = tti.load_tensors(directory)
+        assert callable(loaded["layer.0.weight"]) and callable(loaded["nested"]["layer.1/weight"])  # lazy, as in the reference
+        for name, lazy, fmt, shape in (("layer.0.weight", loaded["layer.0.weight"], O.Bfp8_b, (1, 1, 128, 192)),
+                                       ("layer.1/weight", loaded["nested"]["layer.1/weight"], O.Bfp4_b, (1, 1, 64, 64))):
+            desc = lazy()
+            assert isinstance(desc, B.TilizedTensorDesc if dump == tti.TTIDumpFormat.BACKEND_TILIZED else B.PytorchTensorDesc)
+            q = api.be_api.get_queue_descriptor(name)
+            api.push_input(q, T.pytorch_tensor_to_tensor_desc(desc), True, 1, 0)  # descriptors pass through unchanged
+            assert B.free_tensor(desc) == OK
+            src = params[name] if name in params else params["nested"][name]
+            want = O.unpack_untilize(O.tilize_pack(src.numpy(), fmt), fmt, shape, O.Float16_b)
+            assert np.array_equal(bf16_bits(read(q, pop=False)), want.reshape(-1))
+    finally:
+        api.be_api.finish()  # queue names are reused by the next dump format
+
+
+# ------------------------------------------------------------------------------------------------
+# padding and narrowing at the boundary
+# ------------------------------------------------------------------------------------------------
+
+def test_push_pads_and_get_output_narrows_inside_the_launches(api):
+    say("boundary pad/narrow")
+    q = api.create_queue("ragged", DF.Bfp8_b, (2, 64, 96), num_slots=2)
+    g = torch.Generator().manual_seed(51)
+    x = torch.randn(1, 2, 50, 70, generator=g)
+    assert B.push_input(q, T.pytorch_tensor_to_tensor_desc(x), True, 1, -1) == OK, B.last_error()
+    padded = T.pad_pytorch_tensor_to_buda(x, [])
+    want = O.unpack_untilize(O.tilize_pack(padded.numpy(), O.Bfp8_b), O.Bfp8_b, (1, 2, 64, 96), O.Float32)
+    full = read(q, fp32=True, pop=False)
+    assert full.shape == (1, 2, 64, 96) and np.array_equal(full.numpy().view(np.uint32), want.view(np.uint32))
+    out = B.PytorchTensorDesc()
+    out.format = DF.Float32
+    assert B.get_output(q, out, True, 1, -1, 50, 70) == OK, B.last_error()
+    assert (out.shape, out.strides) == ([1, 2, 50, 70], [2 * 50 * 70 * 4, 50 * 70 * 4, 70 * 4, 4])
+    corner = T.tensor_desc_to_pytorch_tensor(out).clone()
+    B.free_tensor(out)
+    assert torch.equal(corner, full[:, :, :50, :70])
+    assert B.get_output(q, B.PytorchTensorDesc(), True, 1, -1, 20, 70) == ERR and "cannot narrow" in B.last_error()
+    assert B.pop_output(q, True, 1) == OK
+    # a shape whose tiles are not the entry's is still refused
+    assert B.push_input(q, T.pytorch_tensor_to_tensor_desc(torch.zeros(1, 2, 30, 70)), True, 1, -1) == ERR
+    # replicate: a row vector broadcast through its tile, as pad_pytorch_tensor_to_buda does for tile-broadcast dims
+    qb = api.create_queue("bcast_row", DF.Float16_b, (1, 32, 96), 1, RAM)
+    row = torch.randn(1, 1, 1, 70, generator=g).bfloat16()
+    assert B.push_input(qb, T.pytorch_tensor_to_tensor_desc(row), True, 1, 0, True, False) == OK, B.last_error()
+    assert torch.equal(read(qb, pop=False), T.pad_pytorch_tensor_to_buda(row, [-2]))
+    assert B.push_input(qb, T.pytorch_tensor_to_tensor_desc(torch.zeros(1, 1, 2, 70).bfloat16()), True, 1, 0, True, False) == ERR
+    assert "broadcast to tile dim" in B.last_error()
+    # the Python loop: broadcast dims per input, narrowing by original shape
+    api.push_to_queues([qb], [row[0, 0]], single_input=True, tile_broadcast_dims=[[-2]])
+    (y,) = api.read_queues([qb], [(1, 70)], single_output=True, has_microbatch_dim=False)
+    assert y.shape == (1, 70) and torch.equal(y, row[0, 0])
+
+
+def test_pad_to_buda_shape_twin():
+    """pybuda/csrc/tt_torch_device/tt_device.cpp:153-189 on a strided host tensor; align_up_tile: tt_device.hpp:205-210."""
+    assert [B.align_up_tile(d) for d in (1, 31, 32, 33, 64, 1028)] == [32, 32, 32, 64, 64, 1056]
+    base = torch.arange(3 * 50 * 140, dtype=torch.float32).reshape(3, 50, 140)
+    view = base[:, :, ::2]  # [3, 50, 70], column stride two elements
+    d = B.PytorchTensorDesc(view, 4, DF.Float32, 3, [1, 3, 50, 70], [0] + [s * 4 for s in view.stride()])
+    p = B.pad_to_buda_shape(d)
+    assert (p.shape, p.strides, p.dim, p.format) == ([1, 3, 64, 96], [3 * 64 * 96 * 4, 64 * 96 * 4, 96 * 4, 4], 4, DF.Float32)
+    got = T.tensor_desc_to_pytorch_tensor(p).clone()
+    assert B.free_tensor(p) == OK
+    assert torch.equal(got, torch.nn.functional.pad(view, (0, 26, 0, 14)).reshape(1, 3, 64, 96))
+
+
+# ------------------------------------------------------------------------------------------------
+# device-resident sources, overlap on one queue, pools
+# ------------------------------------------------------------------------------------------------
+
+def test_device_tensor_still_being_written_when_it_is_pushed(api):
+    """The source of a push may be a device tensor whose producer kernels are still queued on another stream (torch's);
+    the boundary must not read it before they finish.  A long chain of torch work ends in the tensor, and push_input is
+    called with no synchronization in between."""
+    say("producer ordering")
+    q = api.create_queue("late_src", DF.Bfp8_b, (1, 2048, 2048), num_slots=1)
+    g = torch.Generator(device="cuda").manual_seed(61)
+    a = torch.randn(4096, 4096, generator=g, device="cuda")
+    x = torch.zeros(1, 1, 2048, 2048, device="cuda")
+    torch.cuda.synchronize()
+    acc = a
+    for _ in range(40):            # a few tens of milliseconds of queued matmuls ...
+        acc = (acc @ a) * 1e-2
+        acc = acc / acc.abs().max()
+    x.copy_(acc[:2048, :2048].reshape(1, 1, 2048, 2048))  # ... whose result lands in x last
+    desc = B.PytorchTensorDesc(x, 4, DF.Float32, 4, list(x.shape), [s * 4 for s in x.stride()])
+    assert B.push_input(q, desc, True, 1, -1) == OK, B.last_error()
+    want = O.unpack_untilize(O.tilize_pack(x.cpu().numpy(), O.Bfp8_b, nthreads=8), O.Bfp8_b, (1, 1, 2048, 2048), O.Float16_b)
+    assert float(x.abs().max()) > 0
+    assert np.array_equal(bf16_bits(read(q)), want.reshape(-1))
+
+
+def test_pusher_and_reader_of_one_queue_overlap(api):
+    """The queue's lock covers the ring's bookkeeping only: two pushers and a reader work on one queue at the same time
+    (the count of conversions in flight reaches two or more), entries arrive whole and in the order of the reservations."""
+    say("overlap on one queue")
+    shape = (1, 4096, 4096)  # 32 MiB of bf16 per entry: conversions long enough to meet
+    q = api.create_queue("busy", DF.Bfp8_b, shape, num_slots=4)
+    rounds = 6
+    data = [[torch.full((1, *shape), float(10 * p + r + 1)).bfloat16() for r in range(rounds)] for p in range(2)]
+    errors, seen = [], []
+    start = threading.Barrier(3)
+
+    def pusher(p):
+        start.wait()
+        for r in range(rounds):
+            st = TIMEOUT
+            for _ in range(60):
+                st = B.push_input(q, T.pytorch_tensor_to_tensor_desc(data[p][r]), True, 1, -1)
+                if st != TIMEOUT:
+                    break
+            if st != OK:
+                errors.append(("push", p, r, st, B.last_error()))
+                return
+
+    def reader():
+        start.wait()
+        for _ in range(2 * rounds):
+            out = B.PytorchTensorDesc()
+            st = TIMEOUT
+            for _ in range(60):
+                st = B.get_output(q, out, True, 1, -1)
+                if st != TIMEOUT:
+                    break
+            if st != OK:
+                errors.append(("get", st, B.last_error()))
+                return
+            t = T.tensor_desc_to_pytorch_tensor(out)
+            lo, hi = float(t.min()), float(t.max())
+            B.free_tensor(out)
+            B.pop_output(q, True, 1)
+            if lo != hi:
+                errors.append(("torn entry", lo, hi))
+            seen.append(lo)
+
+    threads = [threading.Thread(target=pusher, args=(0,)), threading.Thread(target=pusher, args=(1,)), threading.Thread(target=reader)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not errors, errors
+    assert not any(t.is_alive() for t in threads)
+    for p in range(2):  # each pusher's entries come out in the order it pushed them
+        mine = [v for v in seen if int(v - 1) // 10 == p]
+        assert mine == [float(10 * p + r + 1) for r in range(rounds)], seen
+    assert api.be_api.queue_max_in_flight("busy") >= 2
+
+
+def test_steady_state_allocates_nothing(api):
+    """Device staging blocks and pinned host blocks are pooled: after the first round trip of a shape the push / get / free
+    cycle allocates no more of either."""
+    say("pools")
+    q = api.create_queue("steady", DF.Bfp8_b, (1, 512, 512), num_slots=2)
+    x = torch.randn(1, 1, 512, 512)
+    ram = api.create_queue("steady_w", DF.Bfp8_b, (1, 512, 512), 1, RAM)
+    for i in range(6):
+        assert B.push_input(q, T.pytorch_tensor_to_tensor_desc(x), True, 1, -1) == OK
+        read(q)
+        t = B.tilize_tensor(ram, T.pytorch_tensor_to_tensor_desc(x))
+        assert B.free_tensor(t) == OK
+        if i == 1:
+            before = B.pool_allocations()
+    assert B.pool_allocations() == before

@@ -72,14 +72,13 @@ SHAPES = [(1, 1, 32, 32), (1, 1, 64, 96), (2, 3, 32, 544), (1, 2, 96, 288)]
 @pytest.mark.parametrize("fmt", BFP + [F.Float16_b, F.Float32])
 @pytest.mark.parametrize("rounding", [0, 1], ids=["trunc", "nearest"])
 def test_tilize_pack_bit_exact(dtype, fmt, rounding):
-    if fmt == F.Float32 and dtype == np.uint16:
-        pytest.skip("a bf16 source does not fill Float32 tiles")
+    widen = fmt == F.Float32 and dtype == np.uint16  # exact: the Float32 tiles of the same values held as fp32
     rng = np.random.default_rng(1000 + fmt + rounding)
     for shape in SHAPES:
         for kind in ("normal", "scaled", "edge"):
             say("tilize_pack", dtype.__name__, fmt, rounding, shape, kind)
             a = make_input(rng, shape, kind, dtype)
-            want = O.tilize_pack(a, fmt, rounding)
+            want = O.tilize_pack((a.astype(np.uint32) << 16).view(np.float32) if widen else a, fmt, rounding)
             got = to_np(capi.tilize_pack(to_dev(a), fmt, rounding))
             assert got.size == want.size
             assert np.array_equal(got, want), f"{shape} {kind}: first diff at {np.flatnonzero(got != want)[:8]}"
@@ -386,9 +385,13 @@ def test_gemm_kernel_selection_shapes(shape):
     b = torch.from_numpy((rng.standard_normal(N) * 0.05).astype(np.float32)).bfloat16()
     xd, wd, bd = x.to(DEV), torch.from_numpy(wp).to(DEV), b.to(DEV)
     base = x.float() @ wdq
-    for bias, epi in ((None, 0), (b, 0), (b, 1), (None, 2)):
+    b3 = b.float() * 3 + 1e-3  # an fp32 bias that is no bf16 value (TTBFP_EPILOGUE_BIAS_F32): three times a bias, as the accumulate form adds it
+    b3d = b3.to(DEV)
+    for bias, epi in ((None, 0), (b, 0), (b, 1), (None, 2), (b3, 0), (b3, 2)):
         say("gemm shapes", shape, "bias" if bias is not None else "nobias", epi)
         want = base + (bias.float() if bias is not None else 0.0)
+        if bias is b3:
+            bd = b3d
         if epi:  # the two forms of pybuda/pybuda/op/eval/pybuda/eltwise_unary.py:42-49
             want = torch.nn.functional.gelu(want, approximate="tanh" if epi == 2 else "none")
         got32 = capi.gemm_bfp8b(xd, wd, N, bias=bd if bias is not None else None, epilogue=epi, out_dtype=torch.float32).cpu()
@@ -564,7 +567,9 @@ def test_gemm_split_over_k_with_a_workspace(shape, out_dtype):
     ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=DEV)  # NaN patterns: every partial must be written before it is read
     wd = capi.unpack_untilize(wp, F.Bfp8_b, (1, 1, K, N))[0, 0]
     base = x.float() @ wd
-    for epi, b in ((capi.EPILOGUE_NONE, None), (capi.EPILOGUE_NONE, bias), (capi.EPILOGUE_GELU, bias), (capi.EPILOGUE_GELU_TANH, bias)):
+    bias32 = bias.float() * 2 + 1e-3  # an fp32 bias that is no bf16 value
+    for epi, b in ((capi.EPILOGUE_NONE, None), (capi.EPILOGUE_NONE, bias), (capi.EPILOGUE_GELU, bias), (capi.EPILOGUE_GELU_TANH, bias),
+                   (capi.EPILOGUE_GELU, bias32)):
         want = base + (b.float() if b is not None else 0.0)
         if epi != capi.EPILOGUE_NONE:
             want = torch.nn.functional.gelu(want, approximate="tanh" if epi == capi.EPILOGUE_GELU_TANH else "none")

@@ -8,6 +8,7 @@ Layers, bottom up:
   tensor        torch <-> descriptor glue (dtype maps, padding, narrowing)
   backend       push / read / pop loops over the queues
   op            matmul / GELU / FFN with Bfp8_b weights
+  tti           tensor entries of a saved device image (.bin / .tbin payloads and their JSON)
 """
 import os as _os
 
@@ -21,6 +22,6 @@ if not _os.path.exists(_os.path.join(_pkg, "libttbfp.so")):
 import torch as _torch  # noqa: E402,F401
 
 from . import _C  # noqa: E402,F401
-from . import backend, capi, op, tensor  # noqa: E402,F401
+from . import backend, capi, op, tensor, tti  # noqa: E402,F401
 from ._C import DataFormat, MathFidelity  # noqa: E402,F401
 from .capi import DataFormatCode  # noqa: E402,F401

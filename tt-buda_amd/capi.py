@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libttbfp.so")
 SUCCESS, RUNTIME_ERROR, TIMEOUT_ERROR = 0, 1, 2
 ROUND_TRUNCATE, ROUND_NEAREST = 0, 1
 EPILOGUE_NONE, EPILOGUE_GELU, EPILOGUE_GELU_TANH = 0, 1, 2
+EPILOGUE_BIAS_F32 = 0x100  # ORed into the epilogue: the bias vector is fp32
 
 
 class DataFormatCode:
@@ -62,6 +63,7 @@ SYMBOLS = {
     "ttbfp_pointer_is_device": (ctypes.c_int32, [ctypes.c_void_p]),
     "ttbfp_stream_create": (ctypes.c_int32, [ctypes.POINTER(ctypes.c_void_p)]),
     "ttbfp_stream_destroy": (ctypes.c_int32, [ctypes.c_void_p]),
+    "ttbfp_device_synchronize": (ctypes.c_int32, []),
     "ttbfp_stream_synchronize": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_int32]),
     "ttbfp_tilize_pack": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, _U64x4, ctypes.c_uint8,
                                            ctypes.c_int32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
@@ -72,6 +74,10 @@ SYMBOLS = {
                                                  _LAYOUT_P, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
     "ttbfp_unpack_untilize_queue": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, _LAYOUT_P, ctypes.c_uint64,
                                                      ctypes.c_uint8, _U64x4, ctypes.c_void_p, ctypes.c_void_p]),
+    "ttbfp_tilize_pack_padded": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, _U64x4, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint8,
+                                                  ctypes.c_int32, _LAYOUT_P, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
+    "ttbfp_unpack_untilize_narrow": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, _LAYOUT_P, ctypes.c_uint64,
+                                                      ctypes.c_uint8, _U64x4, ctypes.c_void_p, ctypes.c_void_p]),
     "ttbfp_prestride_shape": (ctypes.c_uint64, [ctypes.c_uint32, _U32x4, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32 * 2)]),
     "ttbfp_prestride": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint32, _U32x4, _U64x4, ctypes.c_uint32, ctypes.c_void_p,
                                          ctypes.c_uint64, ctypes.c_void_p]),
@@ -82,6 +88,8 @@ SYMBOLS = {
     "ttbfp_gemm_bfp8b_bf16_ws": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
                                                   ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
                                                   ctypes.c_uint8, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
+    "ttbfp_gemm_f32": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                        ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]),
     "ttbfp_static_scratch_bytes": (ctypes.c_uint64, []),
     "ttbfp_gemm_bfp8b_bf16_static": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
                                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
@@ -142,6 +150,8 @@ def tilize_pack(src, dst_fmt, rounding=ROUND_TRUNCATE, out=None):
     nbytes = packed_size(dst_fmt, src.shape)
     if out is None:
         out = torch.empty(nbytes, dtype=torch.uint8, device=src.device)
+    else:
+        assert out.is_cuda and out.device == src.device and out.dtype == torch.uint8 and out.is_contiguous(), "out must be a contiguous uint8 device tensor"
     strides = _U64x4(*[s * src.element_size() for s in src.stride()])
     check(lib().ttbfp_tilize_pack(src.data_ptr(), _TORCH_FMT[src.dtype], _U32x4(*src.shape), strides, dst_fmt, rounding,
                                   out.data_ptr(), out.numel(), _stream()))
@@ -151,15 +161,69 @@ def tilize_pack(src, dst_fmt, rounding=ROUND_TRUNCATE, out=None):
 def unpack_untilize(packed, src_fmt, shape, dtype=torch.float32, out=None):
     """uint8 device tensor of tiles -> row-major 4-D device tensor of ``dtype`` (fp32 or bf16; fp16 for the
     formats with a 5-bit exponent)."""
-    assert packed.is_cuda and packed.dtype == torch.uint8
+    assert packed.is_cuda and packed.dtype == torch.uint8 and packed.is_contiguous()
     if out is None:
         out = torch.empty(tuple(shape), dtype=dtype, device=packed.device)
+    else:  # the C ABI takes strides but no size for the destination
+        assert out.is_cuda and out.device == packed.device and tuple(out.shape) == tuple(shape), "out must be a device tensor of the given shape"
+        assert out.dtype in _TORCH_FMT, "unsupported result dtype"
     need = packed_size(src_fmt, shape)
     if packed.numel() < need:
         raise BackendError(RUNTIME_ERROR, f"packed buffer holds {packed.numel()} bytes, {need} needed")
     strides = _U64x4(*[s * out.element_size() for s in out.stride()])
     check(lib().ttbfp_unpack_untilize(packed.data_ptr(), src_fmt, _U32x4(*shape), _TORCH_FMT[out.dtype], strides,
                                       out.data_ptr(), _stream()))
+    return out
+
+
+def _tiled(shape):
+    return (shape[0], shape[1], (shape[2] + 31) // 32 * 32, (shape[3] + 31) // 32 * 32)
+
+
+def tilize_pack_padded(src, dst_fmt, replicate_rows=False, replicate_cols=False, rounding=ROUND_TRUNCATE, layout=None, pitch=None, out=None):
+    """``tilize_pack`` of a 4-D device tensor whose rows / columns need not be multiples of 32: the padding to whole tiles
+    (zeros, or copies of a single row / column with ``replicate_*``) happens inside the launch."""
+    assert src.is_cuda and src.dim() == 4
+    if src.dtype not in _TORCH_FMT:
+        raise BackendError(RUNTIME_ERROR, f"unsupported source dtype {src.dtype}")
+    tiled = _tiled(src.shape)
+    if layout is None:
+        nbytes, pitch = packed_size(dst_fmt, tiled), 0
+    else:
+        per = queue_buffer_bytes(dst_fmt, tiled, layout)
+        pitch = per if pitch is None else pitch
+        nbytes = max(layout.grid_r * layout.grid_c - 1, 0) * pitch + per
+    if out is None:
+        out = torch.zeros(nbytes, dtype=torch.uint8, device=src.device)
+    else:
+        assert out.is_cuda and out.device == src.device and out.dtype == torch.uint8 and out.is_contiguous()
+    strides = _U64x4(*[s * src.element_size() for s in src.stride()])
+    check(lib().ttbfp_tilize_pack_padded(src.data_ptr(), _TORCH_FMT[src.dtype], _U32x4(*src.shape), strides, int(replicate_rows), int(replicate_cols),
+                                         dst_fmt, rounding, ctypes.byref(layout) if layout is not None else None, pitch, out.data_ptr(),
+                                         out.numel(), _stream()))
+    return out
+
+
+def unpack_untilize_narrow(packed, src_fmt, shape, dtype=torch.float32, layout=None, pitch=None, out=None):
+    """``unpack_untilize`` writing only ``shape`` (rows / columns need not be multiples of 32) out of tiles that cover it
+    rounded up: the narrowing happens inside the launch."""
+    assert packed.is_cuda and packed.dtype == torch.uint8 and packed.is_contiguous()
+    tiled = _tiled(shape)
+    if layout is None:
+        need, pitch = packed_size(src_fmt, tiled), 0
+    else:
+        per = queue_buffer_bytes(src_fmt, tiled, layout)
+        pitch = per if pitch is None else pitch
+        need = max(layout.grid_r * layout.grid_c - 1, 0) * pitch + per
+    if packed.numel() < need:
+        raise BackendError(RUNTIME_ERROR, f"packed buffer holds {packed.numel()} bytes, {need} needed")
+    if out is None:
+        out = torch.empty(tuple(shape), dtype=dtype, device=packed.device)
+    else:
+        assert out.is_cuda and out.device == packed.device and tuple(out.shape) == tuple(shape) and out.dtype in _TORCH_FMT
+    strides = _U64x4(*[s * out.element_size() for s in out.stride()])
+    check(lib().ttbfp_unpack_untilize_narrow(packed.data_ptr(), src_fmt, _U32x4(*shape), ctypes.byref(layout) if layout is not None else None,
+                                             pitch, _TORCH_FMT[out.dtype], strides, out.data_ptr(), _stream()))
     return out
 
 
@@ -177,6 +241,8 @@ def tilize_pack_queue(src, dst_fmt, layout, pitch=None, rounding=ROUND_TRUNCATE,
     pitch = per if pitch is None else pitch
     if out is None:
         out = torch.zeros(max(layout.grid_r * layout.grid_c - 1, 0) * pitch + per, dtype=torch.uint8, device=src.device)
+    else:
+        assert out.is_cuda and out.device == src.device and out.dtype == torch.uint8 and out.is_contiguous(), "out must be a contiguous uint8 device tensor"
     strides = _U64x4(*[s * src.element_size() for s in src.stride()])
     check(lib().ttbfp_tilize_pack_queue(src.data_ptr(), _TORCH_FMT[src.dtype], _U32x4(*src.shape), strides, dst_fmt, rounding,
                                         ctypes.byref(layout), pitch, out.data_ptr(), out.numel(), _stream()))
@@ -193,6 +259,8 @@ def unpack_untilize_queue(queue, src_fmt, shape, layout, pitch=None, dtype=torch
         raise BackendError(RUNTIME_ERROR, f"queue memory holds {queue.numel()} bytes, {need} needed")
     if out is None:
         out = torch.empty(tuple(shape), dtype=dtype, device=queue.device)
+    else:
+        assert out.is_cuda and out.device == queue.device and tuple(out.shape) == tuple(shape) and out.dtype in _TORCH_FMT
     strides = _U64x4(*[s * out.element_size() for s in out.stride()])
     check(lib().ttbfp_unpack_untilize_queue(queue.data_ptr(), src_fmt, _U32x4(*shape), ctypes.byref(layout), pitch,
                                             _TORCH_FMT[out.dtype], strides, out.data_ptr(), _stream()))
@@ -218,18 +286,25 @@ def gemm_workspace_bytes(M, N, K):
 
 
 def gemm_bfp8b(x, w_packed, N, bias=None, epilogue=EPILOGUE_NONE, out_dtype=torch.bfloat16, out=None, workspace=None):
-    """Y = epilogue(X @ dequant(W) + bias).  x: [M, K] bf16 device tensor; w_packed: Bfp8_b tiles of W[K, N].
-    ``workspace``: an optional uint8 device tensor of ``gemm_workspace_bytes(M, N, K)`` bytes."""
+    """Y = epilogue(X @ dequant(W) + bias).  x: [M, K] bf16 device tensor; w_packed: Bfp8_b tiles of W[K, N]; bias: [N] in bf16,
+    or in fp32 (the sum of a bias over a weight stack).  ``workspace``: an optional uint8 device tensor of
+    ``gemm_workspace_bytes(M, N, K)`` bytes."""
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.is_contiguous()
     M, K = x.shape
+    assert w_packed.is_cuda and w_packed.dtype == torch.uint8 and w_packed.is_contiguous()
     if w_packed.numel() < packed_size(DataFormatCode.Bfp8_b, (1, 1, K, N)):
         raise BackendError(RUNTIME_ERROR, "packed weight buffer too small for [K, N]")
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    else:  # the C ABI takes no size for y: a wrong one would be an out-of-bounds device write
+        assert out.is_cuda and out.device == x.device and out.is_contiguous() and tuple(out.shape) == (M, N), "out must be a contiguous [M, N] device tensor"
+        assert out.dtype in (torch.bfloat16, torch.float32), "out must be bf16 or fp32"
     if bias is not None:
-        assert bias.dtype == torch.bfloat16 and bias.numel() == N and bias.is_contiguous()
+        assert bias.is_cuda and bias.dtype in (torch.bfloat16, torch.float32) and bias.numel() == N and bias.is_contiguous()
+        if bias.dtype == torch.float32:
+            epilogue |= EPILOGUE_BIAS_F32
     if workspace is not None:
-        assert workspace.is_cuda and workspace.dtype == torch.uint8
+        assert workspace.is_cuda and workspace.dtype == torch.uint8 and workspace.is_contiguous()
         check(lib().ttbfp_gemm_bfp8b_bf16_ws(M, N, K, x.data_ptr(), w_packed.data_ptr(),
                                              bias.data_ptr() if bias is not None else None, epilogue, out.data_ptr(),
                                              _TORCH_FMT[out.dtype], workspace.data_ptr(), workspace.numel(), _stream()))
@@ -237,4 +312,21 @@ def gemm_bfp8b(x, w_packed, N, bias=None, epilogue=EPILOGUE_NONE, out_dtype=torc
     check(lib().ttbfp_gemm_bfp8b_bf16(M, N, K, x.data_ptr(), w_packed.data_ptr(),
                                       bias.data_ptr() if bias is not None else None, epilogue, out.data_ptr(),
                                       _TORCH_FMT[out.dtype], _stream()))
+    return out
+
+
+def gemm_f32(x, w, bias=None, epilogue=EPILOGUE_NONE, out=None):
+    """Y = epilogue(X @ W + bias) on fp32 row-major device tensors: the matmul of the unquantized (full-precision) mode."""
+    assert x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()
+    assert w.is_cuda and w.dtype == torch.float32 and w.dim() == 2 and w.is_contiguous() and w.shape[0] == x.shape[1]
+    M, K = x.shape
+    N = w.shape[1]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    else:
+        assert out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (M, N)
+    if bias is not None:
+        assert bias.is_cuda and bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()
+    check(lib().ttbfp_gemm_f32(M, N, K, x.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None, epilogue,
+                               out.data_ptr(), _stream()))
     return out

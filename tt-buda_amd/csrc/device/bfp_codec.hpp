@@ -296,7 +296,16 @@ __device__ __forceinline__ float gelu_tanh(float x)
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * u));
 }
 
-// epilogue codes of the GEMM entry points: 0 none, 1 GELU (erf form), 2 GELU (tanh form)
+// The `epilogue` argument of the GEMM entry points: the low byte is the activation (0 none, 1 GELU in its erf form, 2 GELU
+// in its tanh form), bit 8 says that the bias vector holds fp32 values instead of bf16 ones.
+constexpr int kEpilogueMask = 0xff, kEpilogueBiasF32 = 0x100;
+
+// element `col` of the bias row: bf16 (the Float16_b tensor the reference broadcasts) or fp32
+__device__ __forceinline__ float load_bias(const uint16_t *bias, uint32_t col, bool f32)
+{
+    return f32 ? ((const float *)bias)[col] : __uint_as_float((uint32_t)bias[col] << 16);
+}
+
 __device__ __forceinline__ float apply_epilogue(int epilogue, float v)
 {
     if (epilogue == 1) return gelu_erf(v);

@@ -90,21 +90,33 @@ const char *fmt_name(uint8_t fmt)
     }
 }
 
-// Common checks of a [w,z,r,c] view; fills g.  itemsize is that of the row-major side.
+uint32_t align_up_tile(uint32_t d) { return (d + 31u) / 32u * 32u; }  // pybuda/csrc/tt_torch_device/tt_device.hpp:205-210
+
+// Common checks of a [w,z,r,c] view; fills g.  itemsize is that of the row-major side.  With `ragged` the rows and
+// columns of the memory need not be multiples of 32: the tiles then cover the shape rounded up (`tiled`), and what lies
+// past the memory is padding (pack) or left out (unpack).
 int32_t check_geom(const char *fn, const uint32_t shape[4], const uint64_t strides[4], uint32_t itemsize,
-                   ttbfp::TensorGeom &g)
+                   ttbfp::TensorGeom &g, bool ragged = false, uint32_t rep_r = 0, uint32_t rep_c = 0, uint32_t tiled[4] = nullptr)
 {
     if (!shape || !strides) return fail("%s: shape and strides must not be NULL", fn);
-    if (shape[2] % 32 || shape[3] % 32)
+    if (!ragged && (shape[2] % 32 || shape[3] % 32))
         return fail("%s: shape [%u,%u,%u,%u]: rows and columns must be multiples of the 32x32 tile", fn, shape[0],
                     shape[1], shape[2], shape[3]);
+    if (ragged && (shape[2] == 0 || shape[3] == 0 || shape[2] > 0xffffffe0u || shape[3] > 0xffffffe0u))
+        return fail("%s: shape [%u,%u,%u,%u]: rows and columns must lie between 1 and 2^32 - 32", fn, shape[0], shape[1], shape[2], shape[3]);
+    if (rep_r > 1 || rep_c > 1) return fail("%s: the replicate flags are 0 or 1", fn);
+    // the reference replicates only a dimension of one (pybuda/pybuda/tensor.py:852-856)
+    if ((rep_r && shape[2] != 1) || (rep_c && shape[3] != 1))
+        return fail("%s: shape [%u,%u,%u,%u]: only a dimension of size 1 can be replicated into its tile", fn, shape[0], shape[1], shape[2], shape[3]);
     for (int i = 0; i < 4; ++i)
         if (strides[i] % itemsize)
             return fail("%s: stride %d (%llu bytes) is not a multiple of the element size %u", fn, i,
                         (unsigned long long)strides[i], itemsize);
-    const uint64_t elems = (uint64_t)shape[0] * shape[1] * shape[2] * shape[3];
+    const uint32_t R = align_up_tile(shape[2]), C = align_up_tile(shape[3]);
+    const uint64_t elems = (uint64_t)shape[0] * shape[1] * R * C;
     if (elems / 1024 * 64 > 0x7fffffffull * 256ull) return fail("%s: tensor too large", fn);
-    g = {shape[0], shape[1], shape[2], shape[3], strides[0], strides[1], strides[2], strides[3]};
+    g = {shape[0], shape[1], R, C, strides[0], strides[1], strides[2], strides[3], shape[2], shape[3], rep_r, rep_c};
+    if (tiled) tiled[0] = shape[0], tiled[1] = shape[1], tiled[2] = R, tiled[3] = C;
     return TTBFP_SUCCESS;
 }
 
@@ -209,6 +221,8 @@ int32_t ttbfp_stream_destroy(void *stream)
     return stream ? hip_status(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy") : TTBFP_SUCCESS;
 }
 
+int32_t ttbfp_device_synchronize(void) { return hip_status(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
+
 int32_t ttbfp_stream_synchronize(void *stream, int32_t timeout_s)
 {
     if (timeout_s <= 0) return hip_status(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
@@ -239,8 +253,7 @@ int32_t check_pack_formats(const char *fn, uint8_t src_fmt, uint8_t dst_fmt, int
     if (ttbfp::is_a_format(dst_fmt) != (src_fmt == ttbfp::kFloat16))
         return fail("%s: %s source with %s destination: Float16 sources go with Float16/Bfp8/Bfp4/Bfp2 only", fn, fmt_name(src_fmt),
                     fmt_name(dst_fmt));
-    if (dst_fmt == ttbfp::kFloat32 && src_fmt != ttbfp::kFloat32)
-        return fail("%s: a Float16_b source cannot fill Float32 tiles", fn);
+    // a Float16_b source widens exactly into Float32 tiles (the full-precision mode of the host layer keeps queues that way)
     if (rounding != TTBFP_ROUND_TRUNCATE && rounding != TTBFP_ROUND_NEAREST)
         return fail("%s: rounding %d is neither truncate (0) nor nearest (1)", fn, rounding);
     return TTBFP_SUCCESS;
@@ -363,6 +376,51 @@ int32_t ttbfp_unpack_untilize_queue(const void *src_dev, uint8_t src_fmt, const 
     return hip_status(ttbfp::launch_unpack_untilize(src_dev, src_fmt, g, dst_fmt, dst_dev, &q, (hipStream_t)stream), fn);
 }
 
+int32_t ttbfp_tilize_pack_padded(const void *src_dev, uint8_t src_fmt, const uint32_t shape[4], const uint64_t strides_bytes[4],
+                                 uint32_t replicate_rows, uint32_t replicate_cols, uint8_t dst_fmt, int32_t rounding,
+                                 const ttbfp_queue_layout *layout, uint64_t buffer_pitch_bytes, void *dst_dev, uint64_t dst_bytes, void *stream)
+{
+    const char *fn = "ttbfp_tilize_pack_padded";
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (int32_t s = check_pack_formats(fn, src_fmt, dst_fmt, rounding)) return s;
+    ttbfp::TensorGeom g;
+    uint32_t tiled[4];
+    if (int32_t s = check_geom(fn, shape, strides_bytes, src_fmt == ttbfp::kFloat32 ? 4 : 2, g, true, replicate_rows, replicate_cols, tiled)) return s;
+    ttbfp::QueueLayout q;
+    uint64_t need;
+    if (layout) {
+        if (int32_t s = check_layout(fn, dst_fmt, tiled, layout, buffer_pitch_bytes, q)) return s;
+        const uint64_t per_buffer = ttbfp_queue_buffer_bytes(dst_fmt, tiled, layout);
+        need = per_buffer ? ((uint64_t)q.grid_r * q.grid_c - 1) * buffer_pitch_bytes + per_buffer : 0;
+    } else {
+        need = ttbfp_packed_size(dst_fmt, tiled);
+    }
+    if (dst_bytes < need)
+        return fail("%s: destination holds %llu bytes, %llu needed", fn, (unsigned long long)dst_bytes, (unsigned long long)need);
+    if (need == 0) return TTBFP_SUCCESS;
+    if (!src_dev || !dst_dev) return fail("%s: NULL device pointer", fn);
+    return hip_status(ttbfp::launch_tilize_pack(src_dev, src_fmt, g, dst_fmt, rounding, dst_dev, layout ? &q : nullptr, (hipStream_t)stream), fn);
+}
+
+int32_t ttbfp_unpack_untilize_narrow(const void *src_dev, uint8_t src_fmt, const uint32_t shape[4], const ttbfp_queue_layout *layout,
+                                     uint64_t buffer_pitch_bytes, uint8_t dst_fmt, const uint64_t dst_strides_bytes[4], void *dst_dev,
+                                     void *stream)
+{
+    const char *fn = "ttbfp_unpack_untilize_narrow";
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (int32_t s = check_unpack_formats(fn, src_fmt, dst_fmt)) return s;
+    ttbfp::TensorGeom g;
+    uint32_t tiled[4];
+    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, dst_fmt == ttbfp::kFloat32 ? 4 : 2, g, true, 0, 0, tiled)) return s;
+    ttbfp::QueueLayout q;
+    if (layout) {
+        if (int32_t s = check_layout(fn, src_fmt, tiled, layout, buffer_pitch_bytes, q)) return s;
+    }
+    if (ttbfp_packed_size(src_fmt, tiled) == 0) return TTBFP_SUCCESS;
+    if (!src_dev || !dst_dev) return fail("%s: NULL device pointer", fn);
+    return hip_status(ttbfp::launch_unpack_untilize(src_dev, src_fmt, g, dst_fmt, dst_dev, layout ? &q : nullptr, (hipStream_t)stream), fn);
+}
+
 uint64_t ttbfp_prestride_shape(uint32_t itemsize, const uint32_t shape[4], uint32_t stride, uint32_t rows_cols[2])
 {
     if (!shape || !stride || (itemsize != 2 && itemsize != 4)) return 0;
@@ -390,7 +448,8 @@ int32_t ttbfp_prestride(const void *src_dev, uint32_t itemsize, const uint32_t s
     if (need == 0) return TTBFP_SUCCESS;
     if (!src_dev || !dst_dev) return fail("%s: NULL device pointer", fn);
     if ((uintptr_t)src_dev % itemsize || (uintptr_t)dst_dev % itemsize) return fail("%s: pointers must be aligned to the element size", fn);
-    const ttbfp::TensorGeom g = {shape[0], shape[1], shape[2], shape[3], strides_bytes[0], strides_bytes[1], strides_bytes[2], strides_bytes[3]};
+    const ttbfp::TensorGeom g = {shape[0], shape[1], shape[2], shape[3], strides_bytes[0], strides_bytes[1], strides_bytes[2], strides_bytes[3],
+                                 shape[2], shape[3], 0, 0};
     return hip_status(ttbfp::launch_prestride(src_dev, itemsize, g, stride, dst_dev, rc[0], rc[1], (hipStream_t)stream), fn);
 }
 
@@ -404,15 +463,17 @@ int32_t check_gemm(const char *fn, uint32_t M, uint32_t N, uint32_t K, const voi
     nothing_to_do = false;
     if (M % 32 || N % 32 || K % 32 || K == 0)
         return fail("%s: M=%u N=%u K=%u must be multiples of 32 (K non-zero)", fn, M, N, K);
-    if (epilogue != TTBFP_EPILOGUE_NONE && epilogue != TTBFP_EPILOGUE_GELU && epilogue != TTBFP_EPILOGUE_GELU_TANH) return fail("%s: unknown epilogue %d", fn, epilogue);
+    const int32_t activation = epilogue & ~TTBFP_EPILOGUE_BIAS_F32;
+    if (activation != TTBFP_EPILOGUE_NONE && activation != TTBFP_EPILOGUE_GELU && activation != TTBFP_EPILOGUE_GELU_TANH) return fail("%s: unknown epilogue %d", fn, epilogue);
     if (y_fmt != ttbfp::kFloat32 && y_fmt != ttbfp::kFloat16_b) return fail("%s: output format %u: must be Float16_b or Float32", fn, y_fmt);
     if (M == 0 || N == 0) {
         nothing_to_do = true;
         return TTBFP_SUCCESS;
     }
     if (!x_dev || !w_dev || !y_dev) return fail("%s: NULL device pointer", fn);
-    if ((uintptr_t)x_dev % 16 || (uintptr_t)w_dev % 16 || (uintptr_t)y_dev % 16 || (uintptr_t)bias_dev % 2)
-        return fail("%s: x, w and y must be 16-byte aligned", fn);
+    if ((uintptr_t)x_dev % 16 || (uintptr_t)w_dev % 16 || (uintptr_t)y_dev % 16 ||
+        (uintptr_t)bias_dev % ((epilogue & TTBFP_EPILOGUE_BIAS_F32) ? 4 : 2))
+        return fail("%s: x, w and y must be 16-byte aligned, the bias to its element size", fn);
     return TTBFP_SUCCESS;
 }
 
@@ -452,6 +513,18 @@ int32_t ttbfp_gemm_bfp8b_bf16_ws(uint32_t M, uint32_t N, uint32_t K, const void 
     if (!panel)
         return hip_status(ttbfp::launch_gemm_bfp8b_splitk(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, (hipStream_t)stream), fn);
     return hip_status(ttbfp::launch_gemm_bfp8b_panel(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, (hipStream_t)stream), fn);
+}
+
+int32_t ttbfp_gemm_f32(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, const void *w_dev, const void *bias_dev, int32_t epilogue,
+                       void *y_dev, void *stream)
+{
+    const char *fn = "ttbfp_gemm_f32";
+    if (K == 0) return fail("%s: K must not be zero", fn);
+    if (epilogue != TTBFP_EPILOGUE_NONE && epilogue != TTBFP_EPILOGUE_GELU && epilogue != TTBFP_EPILOGUE_GELU_TANH) return fail("%s: unknown epilogue %d", fn, epilogue);
+    if (M == 0 || N == 0) return TTBFP_SUCCESS;
+    if (!x_dev || !w_dev || !y_dev) return fail("%s: NULL device pointer", fn);
+    if ((uintptr_t)x_dev % 4 || (uintptr_t)w_dev % 4 || (uintptr_t)y_dev % 4 || (uintptr_t)bias_dev % 4) return fail("%s: pointers must be 4-byte aligned", fn);
+    return hip_status(ttbfp::launch_gemm_f32(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, (hipStream_t)stream), fn);
 }
 
 uint64_t ttbfp_static_scratch_bytes(void) { return TTBFP_STATIC_SCRATCH_BYTES; }

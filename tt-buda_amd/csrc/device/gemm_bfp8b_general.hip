@@ -38,7 +38,7 @@ template <int EPILOGUE, typename OutT>
 __global__ __launch_bounds__(256) void gemm_bfp8b_general_kernel(uint32_t M, uint32_t N, uint32_t K,
                                                          const uint16_t *__restrict__ X,
                                                          const uint8_t *__restrict__ Wp,
-                                                         const uint16_t *__restrict__ bias, OutT *__restrict__ Y)
+                                                         const uint16_t *__restrict__ bias, int bias_f32, OutT *__restrict__ Y)
 {
     __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDK];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * LDK];
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void gemm_bfp8b_general_kernel(uint32_t M, uin
         for (int nb = 0; nb < 2; ++nb) {
             const uint32_t col = n0 + wn * 64 + nb * 32 + (lane & 31);
             if (col >= N) continue;
-            const float bv = bias ? __uint_as_float((uint32_t)bias[col] << 16) : 0.0f;
+            const float bv = bias ? load_bias(bias, col, bias_f32) : 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t row = m0 + wm * 64 + mb * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
@@ -157,13 +157,13 @@ __global__ __launch_bounds__(256) void gemm_bfp8b_general_kernel(uint32_t M, uin
 }
 
 template <int EPILOGUE, typename OutT>
-hipError_t launch(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, void *y,
+hipError_t launch(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int bias_f32, void *y,
                   hipStream_t stream)
 {
     dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
     if (grid.y > 65535u) return hipErrorInvalidValue;
     hipLaunchKernelGGL((gemm_bfp8b_general_kernel<EPILOGUE, OutT>), grid, dim3(256), 0, stream, M, N, K, (const uint16_t *)x,
-                       (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
+                       (const uint8_t *)w, (const uint16_t *)bias, bias_f32, (OutT *)y);
     return hipGetLastError();
 }
 
@@ -173,14 +173,16 @@ hipError_t launch_gemm_bfp8b_general(uint32_t M, uint32_t N, uint32_t K, const v
                              int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
 {
     if (M == 0 || N == 0) return hipSuccess;
+    const int bias_f32 = epilogue & kEpilogueBiasF32;
+    epilogue &= kEpilogueMask;
     if (y_fmt == kFloat32)
-        return epilogue == 2   ? launch<2, float>(M, N, K, x, w, bias, y, stream)
-               : epilogue == 1 ? launch<1, float>(M, N, K, x, w, bias, y, stream)
-                               : launch<0, float>(M, N, K, x, w, bias, y, stream);
+        return epilogue == 2   ? launch<2, float>(M, N, K, x, w, bias, bias_f32, y, stream)
+               : epilogue == 1 ? launch<1, float>(M, N, K, x, w, bias, bias_f32, y, stream)
+                               : launch<0, float>(M, N, K, x, w, bias, bias_f32, y, stream);
     if (y_fmt == kFloat16_b)
-        return epilogue == 2   ? launch<2, uint16_t>(M, N, K, x, w, bias, y, stream)
-               : epilogue == 1 ? launch<1, uint16_t>(M, N, K, x, w, bias, y, stream)
-                               : launch<0, uint16_t>(M, N, K, x, w, bias, y, stream);
+        return epilogue == 2   ? launch<2, uint16_t>(M, N, K, x, w, bias, bias_f32, y, stream)
+               : epilogue == 1 ? launch<1, uint16_t>(M, N, K, x, w, bias, bias_f32, y, stream)
+                               : launch<0, uint16_t>(M, N, K, x, w, bias, bias_f32, y, stream);
     return hipErrorInvalidValue;
 }
 

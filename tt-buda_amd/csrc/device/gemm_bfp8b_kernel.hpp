@@ -529,14 +529,14 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     static_for<MB * NB>([&](auto bc) {
         constexpr int BLK = decltype(bc)::value, mb = BLK / NB, nb = BLK % NB;
         const uint32_t col = n0 + wn * (BN / S::WN) + nb * 32 + (lane & 31);
-        const float bv = bias ? __uint_as_float((uint32_t)bias[col] << 16) : 0.0f;
+        const float bv = bias ? load_bias(bias, col, epilogue & kEpilogueBiasF32) : 0.0f;
         const uint32_t row0 = m0 + wm * (BM / S::WM) + mb * 32 + (lane >> 5) * 4;
         OutT *yp = Y + (uint64_t)row0 * N + col;
         static_for<16>([&](auto rc) {
             constexpr int r = decltype(rc)::value;
             constexpr uint32_t rr = (r >> 2) * 8 + (r & 3);  // row inside the block, before the lane's 4-row offset
             float v = accumulator_read<16 * BLK + r, ALL_AGPRS>() + bv;
-            v = apply_epilogue(epilogue, v);  // uniform branches
+            v = apply_epilogue(epilogue & kEpilogueMask, v);  // uniform branches
             if constexpr (sizeof(OutT) == 4)
                 yp[(uint64_t)rr * N] = v;
             else

@@ -55,7 +55,7 @@ template <int RT, int EPILOGUE, typename OutT>
 __global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_kernel(uint32_t N, uint32_t K,
                                                                         const uint16_t *__restrict__ X,
                                                                         const uint8_t *__restrict__ Wp,
-                                                                        const uint16_t *__restrict__ bias,
+                                                                        const uint16_t *__restrict__ bias, int bias_f32,
                                                                         OutT *__restrict__ Y)
 {
     constexpr int kWaves = Skinny<RT>::kWaves;
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_ker
         float v = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) v += ((const float *)(lds + w * kRegion))[row * 17 + c];
-        if (bias) v += __uint_as_float((uint32_t)bias[col] << 16);
+        if (bias) v += load_bias(bias, col, bias_f32);
         v = apply_epilogue(EPILOGUE, v);
         if constexpr (sizeof(OutT) == 4)
             Y[(uint64_t)row * N + col] = v;
@@ -207,14 +207,14 @@ __global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_ker
 }
 
 template <int RT, int EPILOGUE, typename OutT>
-hipError_t launch(uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, void *y, hipStream_t stream)
+hipError_t launch(uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int bias_f32, void *y, hipStream_t stream)
 {
     constexpr uint32_t smem = Skinny<RT>::kWaves * Skinny<RT>::kRegion;
     auto kernel = gemm_bfp8b_skinny_kernel<RT, EPILOGUE, OutT>;
     static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (attr != hipSuccess) return attr;
     hipLaunchKernelGGL(kernel, dim3(N / kTile * 2), dim3(64 * Skinny<RT>::kWaves), smem, stream, N, K, (const uint16_t *)x,
-                       (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
+                       (const uint8_t *)w, (const uint16_t *)bias, bias_f32, (OutT *)y);
     return hipGetLastError();
 }
 
@@ -222,14 +222,16 @@ template <int RT>
 hipError_t launch_rows(uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue, void *y, uint8_t y_fmt,
                        hipStream_t stream)
 {
+    const int bias_f32 = epilogue & kEpilogueBiasF32;
+    epilogue &= kEpilogueMask;
     if (y_fmt == kFloat32)
-        return epilogue == 2   ? launch<RT, 2, float>(N, K, x, w, bias, y, stream)
-               : epilogue == 1 ? launch<RT, 1, float>(N, K, x, w, bias, y, stream)
-                               : launch<RT, 0, float>(N, K, x, w, bias, y, stream);
+        return epilogue == 2   ? launch<RT, 2, float>(N, K, x, w, bias, bias_f32, y, stream)
+               : epilogue == 1 ? launch<RT, 1, float>(N, K, x, w, bias, bias_f32, y, stream)
+                               : launch<RT, 0, float>(N, K, x, w, bias, bias_f32, y, stream);
     if (y_fmt == kFloat16_b)
-        return epilogue == 2   ? launch<RT, 2, uint16_t>(N, K, x, w, bias, y, stream)
-               : epilogue == 1 ? launch<RT, 1, uint16_t>(N, K, x, w, bias, y, stream)
-                               : launch<RT, 0, uint16_t>(N, K, x, w, bias, y, stream);
+        return epilogue == 2   ? launch<RT, 2, uint16_t>(N, K, x, w, bias, bias_f32, y, stream)
+               : epilogue == 1 ? launch<RT, 1, uint16_t>(N, K, x, w, bias, bias_f32, y, stream)
+                               : launch<RT, 0, uint16_t>(N, K, x, w, bias, bias_f32, y, stream);
     return hipErrorInvalidValue;
 }
 

@@ -33,8 +33,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(uint64_t quads, uint
     const uint32_t col = (uint32_t)((q * 4) % N);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        if (bias) r[i] += __uint_as_float((uint32_t)bias[col + i] << 16);
-        r[i] = apply_epilogue(epilogue, r[i]);
+        if (bias) r[i] += load_bias(bias, col + i, epilogue & kEpilogueBiasF32);
+        r[i] = apply_epilogue(epilogue & kEpilogueMask, r[i]);
     }
     if constexpr (sizeof(OutT) == 4) {
         *(float4 *)(Y + q * 4) = make_float4(r[0], r[1], r[2], r[3]);

@@ -7,10 +7,18 @@
 namespace ttbfp {
 
 // Row-major [W,Z,R,C] tensor view; strides in bytes, outermost first (tt_PytorchTensorDesc,
-// pybuda/csrc/backend_api/backend_api.cpp:489-560).  R and C are multiples of 32.
+// pybuda/csrc/backend_api/backend_api.cpp:489-560).  R and C are multiples of 32: the extent of the tiles.
+// The memory itself may hold fewer rows and columns, Rl x Cl (the tensor before pad_pytorch_tensor_to_buda,
+// pybuda/pybuda/tensor.py:805-877): packing reads rows >= Rl / columns >= Cl as zeros, or as the last row / column where
+// rep_r / rep_c is set (the reference's "replicate" mode, used for a dimension of one that is broadcast to a tile);
+// unpacking writes the Rl x Cl corner only (narrow_buda_tensor_to_pytorch, tensor.py:879-954).  Rl == R and Cl == C:
+// nothing to pad or narrow.
 struct TensorGeom {
     uint32_t W, Z, R, C;
     uint64_t s0, s1, s2, s3;
+    uint32_t Rl, Cl;
+    uint32_t rep_r, rep_c;
+    bool padded() const { return Rl != R || Cl != C; }
 };
 
 struct QueueLayout;  // queue_layout.hpp
@@ -30,6 +38,10 @@ hipError_t launch_prestride(const void *src, uint32_t itemsize, const TensorGeom
 
 hipError_t launch_gemm_bfp8b(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
                              int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
+
+// Plain fp32 GEMM on row-major operands with an fp32 bias row: the matmul of the full-precision (unquantized) mode.
+hipError_t launch_gemm_f32(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue, void *y,
+                           hipStream_t stream);
 
 // Two-pass form for large M with a caller's workspace: W is converted once into a bf16 panel, then the MFMA kernel
 // runs on that.  gemm_bfp8b_panel_bytes is the workspace it needs, 0 when the fused kernel is the better choice.

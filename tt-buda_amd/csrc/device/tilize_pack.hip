@@ -71,7 +71,9 @@ __device__ __forceinline__ void lds_store(uint8_t *p, uint64_t v)
 // sides instead of one column strip (which would camp on a few HBM channels).
 // QUEUE: the tiles go to their slots of a queue's per-core buffers instead of one linear run; a
 // tile stays one contiguous piece, so only the write-out changes.
-template <typename SrcT, uint8_t DST, int ROUNDING, bool QUEUE>
+// PAD: the memory holds g.Rl x g.Cl (g.Cl a multiple of the elements a lane loads); rows and chunks past that are read from
+// the last row / chunk inside (so that every load stays unconditional) and then zeroed, or kept where g.rep_r says so.
+template <typename SrcT, uint8_t DST, int ROUNDING, bool QUEUE, bool PAD>
 __global__ __launch_bounds__(256) void tilize_pack_rows(const uint8_t *__restrict__ src, TensorGeom g,
                                                         uint8_t *__restrict__ dst, uint32_t segs, QueueLayout q)
 {
@@ -96,11 +98,22 @@ __global__ __launch_bounds__(256) void tilize_pack_rows(const uint8_t *__restric
     // under a condition make the compiler wait for all outstanding loads at once (vmcnt(0)), two full trips to memory
     // before the first row is touched; unconditional ones are counted exactly, row i is converted while rows
     // i + 1 .. 7 are still in flight.
+    uint4 v[8];
+    if constexpr (PAD) {
+        const bool in_cols = c0 < g.Cl;
+        const uint8_t *col0 = src + w * g.s0 + z * g.s1 + (uint64_t)(in_cols ? c0 : g.Cl - EPL) * sizeof(SrcT);
+        const uint32_t r0 = tr * kTile + wave * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = load_stream(col0 + (uint64_t)min(r0 + i, g.Rl - 1) * g.s2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (!in_cols || (r0 + i >= g.Rl && !g.rep_r)) v[i] = make_uint4(0, 0, 0, 0);
+    } else {
     const uint8_t *row0 = src + w * g.s0 + z * g.s1 + (uint64_t)(tr * kTile + wave * 8) * g.s2 +
                           (uint64_t)(live ? c0 : g.C - EPL) * sizeof(SrcT);
-    uint4 v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = load_stream(row0 + i * g.s2);
+    }
     if constexpr (QUEUE) {
         if (threadIdx.x < SEG_TILES && tile0 + threadIdx.x < tiles_c) tile_dst[threadIdx.x] = tile_offset(q, w, z, tr, tile0 + threadIdx.x);
     }
@@ -152,7 +165,7 @@ __global__ __launch_bounds__(256) void tilize_pack_rows(const uint8_t *__restric
                 if (col_in_face == 0) tile_img[face_row] = (uint8_t)(is_a_format(DST) && e ? e - kHalfExponentRebase : e);
             }
         } else if constexpr (DST == kFloat32) {
-            static_assert(sizeof(SrcT) == 4 || DST != kFloat32, "bf16 -> Float32 tiles is not a push conversion");
+            static_assert(sizeof(SrcT) == 4, "16-bit sources reach Float32 tiles through the general kernel only");
             if (live) *(uint4 *)(tile_img + (face_row * 16 + col_in_face) * 4) = v[i];
         } else {  // Float16_b tiles, or Float16 tiles from a half source
             if constexpr (sizeof(SrcT) == 2) {
@@ -214,17 +227,23 @@ __global__ __launch_bounds__(256) void tilize_pack_blocks(const uint8_t *__restr
     const uint32_t face = face_row / kFace, row = face_row % kFace;
     const uint32_t r = tr * kTile + (face / 2) * kFace + row;
     const uint32_t c = tc * kTile + (face % 2) * kFace;
-    const uint8_t *p = src + w * g.s0 + z * g.s1 + (uint64_t)r * g.s2 + (uint64_t)c * g.s3;
+    // rows and columns past the memory's Rl x Cl: the last one inside where the replicate mode says so, else zeros
+    const bool row_inside = r < g.Rl || g.rep_r;
+    const uint8_t *p = src + w * g.s0 + z * g.s1 + (uint64_t)min(r, g.Rl - 1) * g.s2;
     uint32_t bits[16];
+    uint16_t raw[16];  // the half itself, for Float16 tiles
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
+        const bool inside = row_inside && (c + j < g.Cl || g.rep_c);
+        const uint8_t *e = p + (uint64_t)min(c + j, g.Cl - 1) * g.s3;
         if (sizeof(SrcT) == 4)
-            bits[j] = (uint32_t)p[j * g.s3] | (uint32_t)p[j * g.s3 + 1] << 8 | (uint32_t)p[j * g.s3 + 2] << 16 |
-                      (uint32_t)p[j * g.s3 + 3] << 24;
-        else if (std::is_same<SrcT, half_t>::value)
-            bits[j] = half_to_f32_pattern((uint32_t)p[j * g.s3] | (uint32_t)p[j * g.s3 + 1] << 8);
-        else
-            bits[j] = (uint32_t)p[j * g.s3] << 16 | (uint32_t)p[j * g.s3 + 1] << 24;
+            bits[j] = (uint32_t)e[0] | (uint32_t)e[1] << 8 | (uint32_t)e[2] << 16 | (uint32_t)e[3] << 24;
+        else if (std::is_same<SrcT, half_t>::value) {
+            raw[j] = inside ? (uint16_t)((uint32_t)e[0] | (uint32_t)e[1] << 8) : (uint16_t)0;
+            bits[j] = half_to_f32_pattern(raw[j]);
+        } else
+            bits[j] = (uint32_t)e[0] << 16 | (uint32_t)e[1] << 24;
+        if (!inside) bits[j] = 0;
     }
     uint8_t *tile_out = dst + (QUEUE ? tile_offset(q, w, z, tr, tc) : tile * TB);
     if constexpr (QUEUE) {
@@ -250,8 +269,7 @@ __global__ __launch_bounds__(256) void tilize_pack_blocks(const uint8_t *__restr
         for (int j = 0; j < 16; ++j) ((uint32_t *)tile_out)[face_row * 16 + j] = bits[j];
     } else if constexpr (std::is_same<SrcT, half_t>::value) {  // Float16 tiles: the half itself
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-            ((uint16_t *)tile_out)[face_row * 16 + j] = (uint16_t)((uint32_t)p[j * g.s3] | (uint32_t)p[j * g.s3 + 1] << 8);
+        for (int j = 0; j < 16; ++j) ((uint16_t *)tile_out)[face_row * 16 + j] = raw[j];
     } else {
 #pragma unroll
         for (int j = 0; j < 16; ++j)
@@ -265,7 +283,9 @@ __global__ __launch_bounds__(256) void tilize_pack_blocks(const uint8_t *__restr
 // fp32 sources 7-8 % likewise); a small grid wants them all, to cover its ramp and its tail.
 inline uint32_t pack_resident(uint64_t workgroups) { return workgroups >= TTBFP_RESIDENT_MIN_GRID ? TTBFP_PACK_RESIDENT : 8; }
 
-template <typename SrcT, uint8_t DST, int ROUNDING, bool QUEUE>
+// ROWS_OK = false: the pair has no fast kernel (a 16-bit source widened into Float32 tiles: the full-precision mode of the
+// host layer, not a conversion of the hot path) and always takes the general one.
+template <typename SrcT, uint8_t DST, int ROUNDING, bool QUEUE, bool ROWS_OK = true>
 hipError_t launch_kernel(const void *src, const TensorGeom &g, void *dst, const QueueLayout &q, hipStream_t stream)
 {
     const uint32_t tiles_r = g.R / kTile, tiles_c = g.C / kTile;
@@ -275,10 +295,22 @@ hipError_t launch_kernel(const void *src, const TensorGeom &g, void *dst, const 
                          g.s0 % 16 == 0 && g.s1 % 16 == 0 && g.s2 % 16 == 0 && (!QUEUE || q.buffer_pitch % 16 == 0);
     constexpr int SEG_TILES = 64 * Chunk<SrcT>::kElems / kTile;
     const uint32_t segs = (tiles_c + SEG_TILES - 1) / SEG_TILES;
-    if (aligned && bands * segs <= 0x7fffffffull) {
-        hipLaunchKernelGGL((tilize_pack_rows<SrcT, DST, ROUNDING, QUEUE>), dim3((uint32_t)(bands * segs)), dim3(256), resident_cap_bytes(SEG_TILES * tile_bytes(DST), pack_resident(bands * segs)), stream,
-                           (const uint8_t *)src, g, (uint8_t *)dst, segs, q);
-    } else {
+    // padding on the fast path: whole chunks only, and a replicated column is a column of one element
+    const bool pad_ok = g.Cl % Chunk<SrcT>::kElems == 0 && !(g.rep_c && g.Cl != g.C);
+    bool launched = false;
+    if constexpr (ROWS_OK) {
+        if (aligned && bands * segs <= 0x7fffffffull && (!g.padded() || pad_ok)) {
+            const uint32_t lds_cap = resident_cap_bytes(SEG_TILES * tile_bytes(DST), pack_resident(bands * segs));
+            if (g.padded())
+                hipLaunchKernelGGL((tilize_pack_rows<SrcT, DST, ROUNDING, QUEUE, true>), dim3((uint32_t)(bands * segs)), dim3(256), lds_cap, stream,
+                                   (const uint8_t *)src, g, (uint8_t *)dst, segs, q);
+            else
+                hipLaunchKernelGGL((tilize_pack_rows<SrcT, DST, ROUNDING, QUEUE, false>), dim3((uint32_t)(bands * segs)), dim3(256), lds_cap, stream,
+                                   (const uint8_t *)src, g, (uint8_t *)dst, segs, q);
+            launched = true;
+        }
+    }
+    if (!launched) {
         const uint64_t nblocks = bands * tiles_c * 64;
         const uint64_t grid = (nblocks + 255) / 256;
         if (grid > 0x7fffffffull) return hipErrorInvalidValue;
@@ -288,11 +320,11 @@ hipError_t launch_kernel(const void *src, const TensorGeom &g, void *dst, const 
     return hipGetLastError();
 }
 
-template <typename SrcT, uint8_t DST, int ROUNDING>
+template <typename SrcT, uint8_t DST, int ROUNDING, bool ROWS_OK = true>
 hipError_t launch(const void *src, const TensorGeom &g, void *dst, const QueueLayout *q, hipStream_t stream)
 {
-    if (q) return launch_kernel<SrcT, DST, ROUNDING, true>(src, g, dst, *q, stream);
-    return launch_kernel<SrcT, DST, ROUNDING, false>(src, g, dst, QueueLayout{}, stream);
+    if (q) return launch_kernel<SrcT, DST, ROUNDING, true, ROWS_OK>(src, g, dst, *q, stream);
+    return launch_kernel<SrcT, DST, ROUNDING, false, ROWS_OK>(src, g, dst, QueueLayout{}, stream);
 }
 
 // half sources feed the A family only (pybuda/pybuda/device_connector.py:188-192)
@@ -318,7 +350,7 @@ hipError_t by_format(uint8_t dst_fmt, const void *src, const TensorGeom &g, void
         case kFloat16_b: return launch<SrcT, kFloat16_b, ROUNDING>(src, g, dst, q, s);
         case kFloat32:
             if constexpr (sizeof(SrcT) == 4) return launch<SrcT, kFloat32, ROUNDING>(src, g, dst, q, s);
-            return hipErrorInvalidValue;
+            return launch<SrcT, kFloat32, 0, false>(src, g, dst, q, s);  // exact widening, general kernel only
         default: return hipErrorInvalidValue;
     }
 }

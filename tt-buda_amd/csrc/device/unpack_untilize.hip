@@ -36,7 +36,8 @@ __device__ __forceinline__ uint64_t lds_load(const uint8_t *p)
 // bytes; src 16-byte aligned.  1-D grid of bands x segments, segment index fastest (resident
 // workgroups sweep contiguous memory on both sides).
 // QUEUE: the tiles come from their slots of a queue's per-core buffers; only the read-in changes.
-template <uint8_t SRC, typename DstT, bool QUEUE>
+// NARROW: only the g.Rl x g.Cl corner of every [R, C] slice is written (g.Cl a multiple of the elements a lane stores).
+template <uint8_t SRC, typename DstT, bool QUEUE, bool NARROW>
 __global__ __launch_bounds__(256) void unpack_untilize_rows(const uint8_t *__restrict__ src, TensorGeom g,
                                                             uint8_t *__restrict__ dst, uint32_t segs, QueueLayout q)
 {
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(256) void unpack_untilize_rows(const uint8_t *__res
     __syncthreads();
 
     const uint32_t c0 = tile0 * kTile + lane * EPL;
-    if (c0 >= g.C) return;
+    if (c0 >= (NARROW ? g.Cl : g.C)) return;
     uint8_t *row0 = dst + w * g.s0 + z * g.s1 + (uint64_t)(tr * kTile + wave * 8) * g.s2 + (uint64_t)c0 * sizeof(DstT);
     const uint32_t cc = lane * EPL % kTile;
     const uint32_t col_in_face = cc % kFace;
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(256) void unpack_untilize_rows(const uint8_t *__res
             const uint2 h = *(const uint2 *)(tile_img + (face_row * 16 + col_in_face) * 2);
             out = make_uint4(h.x << 16, h.x & 0xffff0000u, h.y << 16, h.y & 0xffff0000u);
         }
-        store_stream(row0 + i * g.s2, out);
+        if (!NARROW || tr * kTile + rr < g.Rl) store_stream(row0 + i * g.s2, out);
     }
 }
 
@@ -174,10 +175,12 @@ __global__ __launch_bounds__(256) void unpack_untilize_blocks(const uint8_t *__r
     const uint32_t face = face_row / kFace, row = face_row % kFace;
     const uint32_t r = tr * kTile + (face / 2) * kFace + row;
     const uint32_t c = tc * kTile + (face % 2) * kFace;
+    if (r >= g.Rl) return;  // narrowed away
     uint8_t *p = dst + w * g.s0 + z * g.s1 + (uint64_t)r * g.s2 + (uint64_t)c * g.s3;
     const uint8_t *tile_in = src + (QUEUE ? tile_offset(q, w, z, tr, tc) : tile * TB);
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
+        if (c + j >= g.Cl) break;
         uint32_t bits;
         if constexpr (M != 0) {
             constexpr int ROW_BYTES = 16 * (M + 1) / 8;
@@ -222,11 +225,17 @@ hipError_t launch_kernel(const void *src, const TensorGeom &g, void *dst, const 
                          g.s0 % 16 == 0 && g.s1 % 16 == 0 && g.s2 % 16 == 0 && (!QUEUE || q.buffer_pitch % 16 == 0);
     constexpr int SEG_TILES = 64 * (16 / sizeof(DstT)) / kTile;
     const uint32_t segs = (tiles_c + SEG_TILES - 1) / SEG_TILES;
-    if (aligned && bands * segs <= 0x7fffffffull) {
+    const bool narrow_ok = g.Cl % (16 / sizeof(DstT)) == 0;  // whole 16-byte stores only
+    if (aligned && bands * segs <= 0x7fffffffull && (!g.padded() || narrow_ok)) {
         // partial segments take the rolled load loop, one load per thread in flight, which needs every workgroup it can get
         const bool mostly_whole = tiles_c % SEG_TILES == 0 || tiles_c >= 4 * SEG_TILES;
-        hipLaunchKernelGGL((unpack_untilize_rows<SRC, DstT, QUEUE>), dim3((uint32_t)(bands * segs)), dim3(256), resident_cap_bytes(SEG_TILES * tile_bytes(SRC), unpack_resident(mostly_whole ? bands * segs : 0, SEG_TILES * tile_bytes(SRC))), stream,
-                           (const uint8_t *)src, g, (uint8_t *)dst, segs, q);
+        const uint32_t lds_cap = resident_cap_bytes(SEG_TILES * tile_bytes(SRC), unpack_resident(mostly_whole ? bands * segs : 0, SEG_TILES * tile_bytes(SRC)));
+        if (g.padded())
+            hipLaunchKernelGGL((unpack_untilize_rows<SRC, DstT, QUEUE, true>), dim3((uint32_t)(bands * segs)), dim3(256), lds_cap, stream,
+                               (const uint8_t *)src, g, (uint8_t *)dst, segs, q);
+        else
+            hipLaunchKernelGGL((unpack_untilize_rows<SRC, DstT, QUEUE, false>), dim3((uint32_t)(bands * segs)), dim3(256), lds_cap, stream,
+                               (const uint8_t *)src, g, (uint8_t *)dst, segs, q);
     } else {
         const uint64_t nblocks = bands * tiles_c * 64;
         const uint64_t grid = (nblocks + 255) / 256;

@@ -53,92 +53,189 @@ bool queue_format_ok(DataFormat f)
 }
 
 // One stream per calling thread: the boundary is entered concurrently from pusher, feeder and main
-// threads (pybuda/pybuda/device_connector.py:147-175, backend.py:145-189).
-void *thread_stream()
+// threads (pybuda/pybuda/device_connector.py:147-175, backend.py:145-189).  `pending` is set when work may be queued on the
+// stream and cleared by a wait that succeeded: memory that such work reads or writes must not be recycled before.
+struct ThreadStream {
+    void *s = nullptr;
+    bool pending = false;
+    ~ThreadStream()
+    {
+        if (!s) return;
+        ttbfp_stream_synchronize(s, 0);
+        ttbfp_stream_destroy(s);
+    }
+};
+
+ThreadStream &thread_ctx()
 {
-    thread_local void *s = nullptr;
-    if (!s && ttbfp_stream_create(&s) != TTBFP_SUCCESS) s = nullptr;
-    return s;
+    thread_local ThreadStream t;
+    if (!t.s && ttbfp_stream_create(&t.s) != TTBFP_SUCCESS) t.s = nullptr;
+    return t;
 }
 
-// Reusable device staging blocks, so the steady-state push/get path does not hipMalloc.
-class StagingPool {
+// the calling thread's stream, for queueing work on it
+void *thread_stream()
+{
+    ThreadStream &t = thread_ctx();
+    t.pending = true;
+    return t.s;
+}
+
+// waits for the thread's stream (timeout_s <= 0: for as long as it takes)
+DEVICE_STATUS_CODE sync_thread_stream(int timeout_s)
+{
+    ThreadStream &t = thread_ctx();
+    const DEVICE_STATUS_CODE st = from_abi(ttbfp_stream_synchronize(t.s, timeout_s));
+    if (st == DEVICE_STATUS_CODE::Success) t.pending = false;
+    return st;
+}
+
+// After a failure or a timeout work may still be queued: true once nothing on the thread's stream can touch memory any
+// more (the error text of the failure that led here is kept).
+bool drain_thread_stream()
+{
+    ThreadStream &t = thread_ctx();
+    if (!t.pending) return true;
+    const std::string keep = g_last_error;
+    const bool ok = ttbfp_stream_synchronize(t.s, 0) == TTBFP_SUCCESS;
+    g_last_error = keep;
+    if (ok) t.pending = false;
+    return ok;
+}
+
+// Reusable blocks of device memory (staging of sources, results and GEMM operands) and of pinned host memory (what
+// tilize_tensor / get_output hand out), so that the steady-state push / get path allocates nothing.  Sizes are rounded to
+// powers of two up to 64 MiB and to multiples of 16 MiB above, so that a 4 GiB request does not pin 8; blocks that come
+// back while the pool already caches `cap` bytes are freed instead of kept.
+class BlockPool {
    public:
+    using AllocFn = std::int32_t (*)(std::uint64_t, void **);
+    using FreeFn = std::int32_t (*)(void *);
+    BlockPool(AllocFn a, FreeFn f, std::uint64_t cap) : alloc_(a), free_(f), cap_(cap) {}
+
+    static std::uint64_t rounded(std::uint64_t bytes)
+    {
+        constexpr std::uint64_t kBig = 64ull << 20, kStep = 16ull << 20;
+        if (bytes > kBig) return (bytes + kStep - 1) / kStep * kStep;
+        std::uint64_t size = 1 << 16;
+        while (size < bytes) size <<= 1;
+        return size;
+    }
     DEVICE_STATUS_CODE take(std::uint64_t bytes, void **out)
     {
-        std::uint64_t cap = 1 << 16;
-        while (cap < bytes) cap <<= 1;
+        const std::uint64_t size = rounded(bytes);
         {
             std::lock_guard<std::mutex> l(m_);
-            auto &bucket = free_[cap];
+            auto &bucket = free_blocks_[size];
             if (!bucket.empty()) {
                 *out = bucket.back();
                 bucket.pop_back();
+                cached_ -= size;
                 return DEVICE_STATUS_CODE::Success;
             }
         }
-        TT_TRY(from_abi(ttbfp_alloc(cap, out)));
+        TT_TRY(from_abi(alloc_(size, out)));
         std::lock_guard<std::mutex> l(m_);
-        size_of_[*out] = cap;
+        size_of_[*out] = size;
+        allocations_ += 1;
         return DEVICE_STATUS_CODE::Success;
     }
-    void give(void *p)
+    // true if `p` is one of the pool's blocks (it is then back in the pool, or freed)
+    bool give(const void *p)
     {
-        if (!p) return;
+        if (!p) return false;
+        std::uint64_t size;
+        {
+            std::lock_guard<std::mutex> l(m_);
+            auto it = size_of_.find(p);
+            if (it == size_of_.end()) return false;
+            size = it->second;
+            if (cached_ + size <= cap_) {
+                free_blocks_[size].push_back(const_cast<void *>(p));
+                cached_ += size;
+                return true;
+            }
+            size_of_.erase(it);
+        }
+        free_(const_cast<void *>(p));
+        return true;
+    }
+    std::uint64_t allocations()
+    {
         std::lock_guard<std::mutex> l(m_);
-        free_[size_of_[p]].push_back(p);
+        return allocations_;
     }
 
    private:
+    AllocFn alloc_;
+    FreeFn free_;
+    std::uint64_t cap_, cached_ = 0, allocations_ = 0;
     std::mutex m_;
-    std::map<std::uint64_t, std::vector<void *>> free_;
-    std::unordered_map<void *, std::uint64_t> size_of_;
+    std::map<std::uint64_t, std::vector<void *>> free_blocks_;
+    std::unordered_map<const void *, std::uint64_t> size_of_;
 };
 
-StagingPool &staging()
+std::uint64_t pool_cap(const char *env, std::uint64_t fallback)
 {
-    static StagingPool *pool = new StagingPool();  // never destroyed: HIP may be gone at exit
+    const char *v = std::getenv(env);
+    return v && *v ? std::strtoull(v, nullptr, 10) : fallback;
+}
+
+// never destroyed: HIP may be gone when static destructors run
+BlockPool &staging()
+{
+    static BlockPool *pool = new BlockPool(ttbfp_alloc, ttbfp_free, pool_cap("TTBFP_DEVICE_POOL_BYTES", 16ull << 30));
+    return *pool;
+}
+BlockPool &pinned()
+{
+    static BlockPool *pool = new BlockPool(ttbfp_host_alloc, ttbfp_host_free, pool_cap("TTBFP_HOST_POOL_BYTES", 4ull << 30));
     return *pool;
 }
 
-struct Staged {  // RAII return to the pool
+// A staging block for the duration of a call.  It goes back to the pool only once nothing queued on the thread's stream
+// can still use it: after an error or a timeout the stream is drained first, and if even that fails the block is leaked
+// rather than handed to another thread while the GPU may still write it.
+struct Staged {
     void *p = nullptr;
-    ~Staged() { staging().give(p); }
+    ~Staged()
+    {
+        if (p && drain_thread_stream()) staging().give(p);
+    }
 };
 
-// Host memory handed to the caller by tilize_tensor / get_output / debinarize_tensor.
-std::mutex g_host_mutex;
-std::unordered_map<const void *, std::uint64_t> g_host_blocks;
-
-DEVICE_STATUS_CODE host_block(std::uint64_t bytes, void **out)
-{
-    TT_TRY(from_abi(ttbfp_host_alloc(bytes ? bytes : 1, out)));
-    std::lock_guard<std::mutex> l(g_host_mutex);
-    g_host_blocks[*out] = bytes;
-    return DEVICE_STATUS_CODE::Success;
-}
+// Host memory handed to the caller by tilize_tensor / get_output / debinarize_tensor / pad_to_buda_shape: pinned blocks
+// from the pool, given back by free_tensor.
+DEVICE_STATUS_CODE host_block(std::uint64_t bytes, void **out) { return pinned().take(bytes ? bytes : 1, out); }
 
 DEVICE_STATUS_CODE release_host_block(const void *p)
 {
-    {
-        std::lock_guard<std::mutex> l(g_host_mutex);
-        auto it = g_host_blocks.find(p);
-        if (it == g_host_blocks.end()) return DEVICE_STATUS_CODE::Success;  // not ours: the caller's tensor
-        g_host_blocks.erase(it);
-    }
-    return from_abi(ttbfp_host_free(const_cast<void *>(p)));
+    if (!drain_thread_stream()) return DEVICE_STATUS_CODE::RuntimeError;  // a copy into it may be in flight: leak it
+    pinned().give(p);  // not one of ours: the caller's tensor, nothing to do
+    return DEVICE_STATUS_CODE::Success;
 }
 
 // HBM of a queue: buffer b of the grid starts at base + b * pitch and holds the queue's `slots` entries
 // one after another, `entry_bytes` each (that buffer's share of an entry).
+//
+// The mutex guards the ring's bookkeeping only.  A pusher reserves its slots under it, converts into them with the lock
+// released, and publishes them under it again, in the order of the reservations (so that entries become visible in the
+// order their slots lie in the ring); a reader pins the entries it reads (`readers`) and pop_output waits for that pin,
+// so a pusher and a reader of one queue overlap their GPU work, as the reference's callers expect of a boundary they
+// enter without the GIL (pybuda/csrc/backend_api/backend_api.cpp:688-701).
 struct Queue {
     tt_dram_io_desc desc;
+    DataFormat storage = DataFormat::Invalid;  // format of the tiles in HBM: the declared one, or its full-precision stand-in
     ttbfp_queue_layout layout{};
     std::uint8_t *base = nullptr;
     std::uint64_t entry_bytes = 0, pitch = 0;
     std::uint32_t buffers = 1;
     bool row_major = true;  // plain row-major header-less tiles in one buffer
     std::uint32_t slots = 0, wr = 0, rd = 0, count = 0;
+    std::uint32_t reserved = 0;                   // entries being written, behind wr + count
+    std::uint64_t ticket_next = 0, ticket_done = 0;  // reservations handed out / published
+    std::uint32_t readers = 0;                    // get_output calls reading entries right now
+    std::uint32_t in_flight = 0, max_in_flight = 0;  // conversions running outside the lock, and the most there ever were
     std::uint8_t *slot(std::uint32_t s) const { return base + s * entry_bytes; }  // in buffer 0; the others `pitch` apart
     std::uint64_t span(std::uint32_t entries) const { return (buffers - 1) * pitch + entries * entry_bytes; }
     std::mutex m;
@@ -163,11 +260,20 @@ ttbfp_queue_layout layout_of(const tt_dram_io_desc &d)
 }
 
 // One buffer's share of one entry.
-std::uint64_t entry_bytes_of(const tt_dram_io_desc &d)
+std::uint64_t entry_bytes_of(const tt_dram_io_desc &d, DataFormat storage)
 {
     const std::uint32_t shape[4] = {1, d.t, d.rows(), d.cols()};
     const ttbfp_queue_layout l = layout_of(d);
-    return ttbfp_queue_buffer_bytes((std::uint8_t)d.bufq_target_format, shape, &l);
+    return ttbfp_queue_buffer_bytes((std::uint8_t)storage, shape, &l);
+}
+
+// What a queue holds when the backend ignores the precision of data formats (BackendConfig::ignore_data_format_precision,
+// pybuda/csrc/backend_api/backend_api.cpp:261-275: "run backend at full precision"): every format with an 8-bit exponent
+// keeps fp32 tiles, the family with the 5-bit exponent of IEEE half keeps the halves it is fed, raw integers stay raw.
+DataFormat full_precision_of(DataFormat f)
+{
+    if (f == DataFormat::RawUInt32) return f;
+    return a_family(f) ? DataFormat::Float16 : DataFormat::Float32;
 }
 
 // Header-less tiles of one buffer in plain row-major order: what the GEMM reads its weight in.
@@ -178,14 +284,21 @@ bool row_major_order(const tt_dram_io_desc &d)
 }
 
 // tilize+pack `wn` entries of a row-major device tensor into slots slot0.. of a queue, and the reverse.
+// The memory holds rows x cols per slice (0: as many as the entry has); what lies between that and the entry's
+// tile-aligned extent is padding made inside the launch: zeros, or copies of a single row / column (rep_r / rep_c).
 DEVICE_STATUS_CODE pack_into(const Queue &q, std::uint32_t slot0, const std::uint8_t *src, DataFormat src_fmt, std::uint32_t wn,
-                             const std::uint64_t st[4], void *stream)
+                             const std::uint64_t st[4], void *stream, std::uint32_t rows = 0, std::uint32_t cols = 0, bool rep_r = false,
+                             bool rep_c = false)
 {
-    const std::uint32_t shape[4] = {wn, q.desc.t, q.desc.rows(), q.desc.cols()};
+    const std::uint32_t shape[4] = {wn, q.desc.t, rows ? rows : q.desc.rows(), cols ? cols : q.desc.cols()};
+    if (shape[2] != q.desc.rows() || shape[3] != q.desc.cols())
+        return from_abi(ttbfp_tilize_pack_padded(src, (std::uint8_t)src_fmt, shape, st, rep_r, rep_c, (std::uint8_t)q.storage, conversion_rounding(),
+                                                 q.row_major ? nullptr : &q.layout, q.pitch, q.slot(slot0),
+                                                 q.row_major ? wn * q.entry_bytes : q.span(wn), stream));
     if (q.row_major)
-        return from_abi(ttbfp_tilize_pack(src, (std::uint8_t)src_fmt, shape, st, (std::uint8_t)q.desc.bufq_target_format,
+        return from_abi(ttbfp_tilize_pack(src, (std::uint8_t)src_fmt, shape, st, (std::uint8_t)q.storage,
                                           conversion_rounding(), q.slot(slot0), wn * q.entry_bytes, stream));
-    return from_abi(ttbfp_tilize_pack_queue(src, (std::uint8_t)src_fmt, shape, st, (std::uint8_t)q.desc.bufq_target_format,
+    return from_abi(ttbfp_tilize_pack_queue(src, (std::uint8_t)src_fmt, shape, st, (std::uint8_t)q.storage,
                                             conversion_rounding(), &q.layout, q.pitch, q.slot(slot0), q.span(wn), stream));
 }
 
@@ -234,20 +347,117 @@ DEVICE_STATUS_CODE check_source(const tt_PytorchTensorDesc &t, DataFormat dst, c
 }
 
 // `zn` z slices starting at slice z0 of `wn` entries from slot slot0 on -> row-major memory with byte strides st.
+// rows / cols (0: all): only that corner of every slice is written, the narrowing done inside the launch
 DEVICE_STATUS_CODE unpack_from(const Queue &q, std::uint32_t slot0, std::uint32_t wn, std::uint32_t z0, std::uint32_t zn, DataFormat dst_fmt,
-                               const std::uint64_t st[4], void *dst, void *stream)
+                               const std::uint64_t st[4], void *dst, void *stream, std::uint32_t rows = 0, std::uint32_t cols = 0)
 {
-    const std::uint32_t shape[4] = {wn, zn, q.desc.rows(), q.desc.cols()};
+    const std::uint32_t shape[4] = {wn, zn, rows ? rows : q.desc.rows(), cols ? cols : q.desc.cols()};
     const std::uint8_t *src = q.slot(slot0) + z0 * (q.entry_bytes / q.desc.t);  // a buffer holds its z slices one after another
+    if (shape[2] != q.desc.rows() || shape[3] != q.desc.cols())
+        return from_abi(ttbfp_unpack_untilize_narrow(src, (std::uint8_t)q.storage, shape, q.row_major ? nullptr : &q.layout, q.pitch,
+                                                     (std::uint8_t)dst_fmt, st, dst, stream));
     if (q.row_major)
-        return from_abi(ttbfp_unpack_untilize(src, (std::uint8_t)q.desc.bufq_target_format, shape, (std::uint8_t)dst_fmt, st, dst, stream));
-    return from_abi(ttbfp_unpack_untilize_queue(src, (std::uint8_t)q.desc.bufq_target_format, shape, &q.layout, q.pitch,
+        return from_abi(ttbfp_unpack_untilize(src, (std::uint8_t)q.storage, shape, (std::uint8_t)dst_fmt, st, dst, stream));
+    return from_abi(ttbfp_unpack_untilize_queue(src, (std::uint8_t)q.storage, shape, &q.layout, q.pitch,
                                                 (std::uint8_t)dst_fmt, st, dst, stream));
+}
+
+// ---- the ring's bookkeeping: everything below runs with the queue's mutex held only while it touches these fields ----
+
+struct Reservation {
+    std::uint32_t slot0 = 0, n = 0;
+    std::uint64_t ticket = 0;
+    bool ring = false;
+};
+
+// Slots for n entries: the next n free ones of a ring (waits up to timeout_s for space), or slots ram_ptr.. of a RAM.
+DEVICE_STATUS_CODE reserve_write(Queue &q, std::uint32_t n, int timeout_s, int ram_ptr, Reservation &r, const char *fn)
+{
+    std::unique_lock<std::mutex> l(q.m);
+    r.n = n;
+    r.ring = q.desc.io_type == IO_TYPE::Queue;
+    if (r.ring) {
+        if (!wait_until(l, q.cv, timeout_s, [&] { return q.slots - q.count - q.reserved >= n; }))
+            return fail(std::string(fn) + ": queue '" + q.desc.queue_name + "' is full", DEVICE_STATUS_CODE::TimeoutError);
+        r.slot0 = (q.wr + q.reserved) % q.slots;
+        r.ticket = q.ticket_next++;
+        q.reserved += n;
+    } else {
+        r.slot0 = ram_ptr < 0 ? 0 : (std::uint32_t)ram_ptr;
+        if (r.slot0 + n > q.slots) return fail(std::string(fn) + ": ram pointer past the end of '" + q.desc.queue_name + "'");
+    }
+    q.in_flight += 1;
+    q.max_in_flight = std::max(q.max_in_flight, q.in_flight);
+    return DEVICE_STATUS_CODE::Success;
+}
+
+// Makes the reserved entries visible, once every earlier reservation has been.  After a failure the slots are given up
+// again if nobody reserved behind them; otherwise they are published as they are, so that the ring stays whole (a failing
+// HIP call leaves the process without a usable device anyway).
+void publish_write(Queue &q, const Reservation &r, bool ok)
+{
+    std::unique_lock<std::mutex> l(q.m);
+    q.in_flight -= 1;
+    if (r.ring) {
+        q.cv.wait(l, [&] { return q.ticket_done == r.ticket; });
+        q.reserved -= r.n;
+        if (ok || q.ticket_next != r.ticket + 1) {
+            q.wr = (q.wr + r.n) % q.slots;
+            q.count += r.n;
+        }
+        if (!ok && q.ticket_next == r.ticket + 1) q.ticket_next = r.ticket;  // the rollback hands the ticket back too
+        else q.ticket_done += 1;
+    }
+    q.cv.notify_all();
+}
+
+// Pins n entries for reading: the oldest n of a ring (waits up to timeout_s for them; rd_ptr >= 0 names the first slot
+// instead), or slots rd_ptr.. of a RAM.
+DEVICE_STATUS_CODE begin_read(Queue &q, std::uint32_t n, int timeout_s, int rd_ptr, std::uint32_t &slot0, const char *fn)
+{
+    std::unique_lock<std::mutex> l(q.m);
+    if (q.desc.io_type == IO_TYPE::Queue) {
+        if (!wait_until(l, q.cv, timeout_s, [&] { return q.count >= n; }))
+            return fail(std::string(fn) + ": queue '" + q.desc.queue_name + "' is empty", DEVICE_STATUS_CODE::TimeoutError);
+        slot0 = rd_ptr >= 0 ? (std::uint32_t)rd_ptr % q.slots : q.rd;
+    } else {
+        slot0 = rd_ptr < 0 ? 0 : (std::uint32_t)rd_ptr;
+        if (slot0 + n > q.slots) return fail(std::string(fn) + ": read pointer past the end of '" + q.desc.queue_name + "'");
+    }
+    q.readers += 1;
+    q.in_flight += 1;
+    q.max_in_flight = std::max(q.max_in_flight, q.in_flight);
+    return DEVICE_STATUS_CODE::Success;
+}
+
+void end_read(Queue &q)
+{
+    std::lock_guard<std::mutex> l(q.m);
+    q.readers -= 1;
+    q.in_flight -= 1;
+    q.cv.notify_all();
+}
+
+// Releases the oldest n entries of a ring (waits up to timeout_s for them and for readers that still hold them).
+DEVICE_STATUS_CODE release_entries(Queue &q, std::uint32_t n, int timeout_s, const char *fn)
+{
+    std::unique_lock<std::mutex> l(q.m);
+    if (!wait_until(l, q.cv, timeout_s, [&] { return q.count >= n && q.readers == 0; }))
+        return fail(std::string(fn) + ": queue '" + q.desc.queue_name + (q.count >= n ? "' is being read" : "' is empty"),
+                    DEVICE_STATUS_CODE::TimeoutError);
+    q.rd = (q.rd + n) % q.slots;
+    q.count -= n;
+    q.cv.notify_all();
+    return DEVICE_STATUS_CODE::Success;
 }
 
 DEVICE_STATUS_CODE stage_source(const tt_PytorchTensorDesc &t, Staged &staged, const std::uint8_t **dev_src, void *stream)
 {
     if (ttbfp_pointer_is_device(t.ptr)) {
+        // The tensor already lives in HBM.  Which stream produced it is not known here (the descriptor carries a pointer,
+        // nothing else) and this thread's stream is not ordered after any other, so wait for all work on the device first:
+        // the call then sees the tensor as complete as it would see a host tensor.
+        TT_TRY(from_abi(ttbfp_device_synchronize()));
         *dev_src = (const std::uint8_t *)t.ptr;
         return DEVICE_STATUS_CODE::Success;
     }
@@ -271,7 +481,7 @@ int conversion_rounding()
 
 // ---- tt_backend ------------------------------------------------------------------------------
 
-tt_backend::tt_backend(int device) : device_(device)
+tt_backend::tt_backend(int device, const tt_backend_config &config) : device_(device), config_(config)
 {
     static std::mutex m;
     static int counter = 0;
@@ -279,13 +489,20 @@ tt_backend::tt_backend(int device) : device_(device)
     id_ = "hip_backend_" + std::to_string(counter++);
 }
 
-std::shared_ptr<tt_backend> tt_backend::create(int device) { return std::shared_ptr<tt_backend>(new tt_backend(device)); }
+std::shared_ptr<tt_backend> tt_backend::create(int device, const tt_backend_config &config)
+{
+    return std::shared_ptr<tt_backend>(new tt_backend(device, config));
+}
 
 tt_backend::~tt_backend() { finish(); }
 
 DEVICE_STATUS_CODE tt_backend::initialize() { return from_abi(ttbfp_init(device_)); }
 
-DEVICE_STATUS_CODE tt_backend::wait_for_idle() { return from_abi(ttbfp_stream_synchronize(thread_stream(), 0)); }
+DEVICE_STATUS_CODE tt_backend::wait_for_idle()
+{
+    thread_stream();
+    return sync_thread_stream(0);
+}
 
 DEVICE_STATUS_CODE tt_backend::finish()
 {
@@ -332,10 +549,11 @@ tt_dram_io_desc tt_backend::create_queue(const std::string &name, DataFormat for
     d.input_count = input_count;
     d.bufq_target_format = format;
     d.io_type = io_type;
+    q->storage = config_.ignore_data_format_precision ? full_precision_of(format) : format;
     q->layout = layout_of(d);
     q->row_major = row_major_order(d);
     q->buffers = grid_r * grid_c;
-    q->entry_bytes = entry_bytes_of(d);
+    q->entry_bytes = entry_bytes_of(d, q->storage);
     if (q->entry_bytes > 0xffffffffull) throw std::runtime_error("create_queue: one entry exceeds 4 GiB");
     d.bufq_entry_size = (std::uint32_t)q->entry_bytes;
     q->slots = num_slots;
@@ -344,9 +562,13 @@ tt_dram_io_desc tt_backend::create_queue(const std::string &name, DataFormat for
     if (ttbfp_alloc(q->pitch * q->buffers, &base) != TTBFP_SUCCESS)
         throw std::runtime_error(std::string("create_queue: ") + ttbfp_last_error());
     q->base = (std::uint8_t *)base;
-    d.bufq_start_addr_channel.clear();  // one (address, channel) pair per buffer of the grid; the channel is always HBM 0
-    for (std::uint32_t b = 0; b < q->buffers; ++b)
-        d.bufq_start_addr_channel.push_back({(std::uint32_t)((std::uintptr_t)(q->base + b * q->pitch) & 0xffffffffu), 0});
+    // One (address, channel) pair per buffer of the grid.  The reference's pair is 32 + 16 bits wide; an HBM address here
+    // has 48 significant bits, so the pair carries all of it: the low 32 bits as the address, the upper 16 as the channel.
+    d.bufq_start_addr_channel.clear();
+    for (std::uint32_t b = 0; b < q->buffers; ++b) {
+        const std::uint64_t addr = (std::uint64_t)(std::uintptr_t)(q->base + b * q->pitch);
+        d.bufq_start_addr_channel.push_back({(std::uint32_t)(addr & 0xffffffffu), (std::uint16_t)((addr >> 32) & 0xffffu)});
+    }
     {
         std::lock_guard<std::mutex> l(g_registry_mutex);
         if (g_registry.count(key_of(d))) {
@@ -367,6 +589,27 @@ tt_dram_io_desc tt_backend::get_queue_descriptor(const std::string &name) const
     return it->second->desc;
 }
 
+DataFormat tt_backend::queue_storage_format(const std::string &name) const
+{
+    std::lock_guard<std::mutex> l(g_registry_mutex);
+    auto it = g_registry.find(id_ + "/" + name);
+    if (it == g_registry.end()) throw std::runtime_error("queue_storage_format: no queue named '" + name + "'");
+    return it->second->storage;
+}
+
+std::uint32_t tt_backend::queue_max_in_flight(const std::string &name) const
+{
+    std::shared_ptr<Queue> q;
+    {
+        std::lock_guard<std::mutex> l(g_registry_mutex);
+        auto it = g_registry.find(id_ + "/" + name);
+        if (it == g_registry.end()) throw std::runtime_error("queue_max_in_flight: no queue named '" + name + "'");
+        q = it->second;
+    }
+    std::lock_guard<std::mutex> l(q->m);
+    return q->max_in_flight;
+}
+
 DEVICE_STATUS_CODE tt_backend::run_matmul(const std::string &in0, const std::string &weight, const std::string &bias,
                                           const std::string &out, bool gelu, int timeout_s, const std::string &approximate)
 {
@@ -384,58 +627,64 @@ DEVICE_STATUS_CODE tt_backend::run_matmul(const std::string &in0, const std::str
     if (qa->desc.t != 1 || qw->desc.t != 1 || qo->desc.t != 1) return fail("run_matmul: t > 1 is not supported");
     if (qw->desc.rows() != K || qo->desc.rows() != M || qo->desc.cols() != N)
         return fail("run_matmul: queue shapes do not form [M,K] x [K,N] -> [M,N]");
-    if (qw->desc.bufq_target_format != DataFormat::Bfp8_b) return fail("run_matmul: the weight queue must be Bfp8_b");
-    if (!qw->row_major)
-        return fail("run_matmul: the weight queue must hold header-less tiles in row-major order (grid 1x1 and one-tile-high micro "
-                    "blocks in r order, or one micro block per row of the macro block)");
     if (qb && (qb->desc.cols() != N || qb->desc.t != 1)) return fail("run_matmul: bias queue must be [32k, N]");
+    // Full-precision mode: the queues hold unquantized fp32 tiles and the matmul is evaluated on them as they are.
+    const bool full = config_.ignore_data_format_precision;
+    if (full) {
+        for (const auto &q : {qa, qw, qo, qb})
+            if (q && q->storage != DataFormat::Float32) return fail("run_matmul: full-precision mode needs queues with an 8-bit exponent");
+    } else {
+        if (qw->desc.bufq_target_format != DataFormat::Bfp8_b) return fail("run_matmul: the weight queue must be Bfp8_b");
+        if (!qw->row_major)
+            return fail("run_matmul: the weight queue must hold header-less tiles in row-major order (grid 1x1 and one-tile-high micro "
+                        "blocks in r order, or one micro block per row of the macro block)");
+    }
+    const std::uint32_t isz = full ? 4 : 2;
+    const DataFormat act_fmt = full ? DataFormat::Float32 : DataFormat::Float16_b;
 
     void *stream = thread_stream();
-    Staged x, y, b;
-    TT_TRY(staging().take((std::uint64_t)M * K * 2, &x.p));
-    TT_TRY(staging().take((std::uint64_t)M * N * 2, &y.p));
+    Staged x, y, b, w_full, panel;
+    TT_TRY(staging().take((std::uint64_t)M * K * isz, &x.p));
+    TT_TRY(staging().take((std::uint64_t)M * N * isz, &y.p));
 
-    std::uint32_t in_slot;
+    std::uint32_t in_slot = 0;
+    TT_TRY(begin_read(*qa, 1, timeout_s, -1, in_slot, "run_matmul"));
+    struct ReadPin {
+        Queue &q;
+        ~ReadPin() { end_read(q); }
+    } pin{*qa};
     {
-        std::unique_lock<std::mutex> l(qa->m);
-        if (!wait_until(l, qa->cv, timeout_s, [&] { return qa->count >= 1; }))
-            return fail("run_matmul: timed out waiting for an entry in " + in0, DEVICE_STATUS_CODE::TimeoutError);
-        in_slot = qa->rd;
-    }
-    {
-        const std::uint64_t st[4] = {(std::uint64_t)M * K * 2, (std::uint64_t)M * K * 2, (std::uint64_t)K * 2, 2};
-        TT_TRY(unpack_from(*qa, in_slot, 1, 0, 1, DataFormat::Float16_b, st, x.p, stream));
+        const std::uint64_t st[4] = {(std::uint64_t)M * K * isz, (std::uint64_t)M * K * isz, (std::uint64_t)K * isz, isz};
+        TT_TRY(unpack_from(*qa, in_slot, 1, 0, 1, act_fmt, st, x.p, stream));
     }
     const void *bias_dev = nullptr;
     if (qb) {
         const std::uint32_t R = qb->desc.rows();
-        TT_TRY(staging().take((std::uint64_t)R * N * 2, &b.p));
-        const std::uint64_t st[4] = {(std::uint64_t)R * N * 2, (std::uint64_t)R * N * 2, (std::uint64_t)N * 2, 2};
-        TT_TRY(unpack_from(*qb, 0, 1, 0, 1, DataFormat::Float16_b, st, b.p, stream));
+        TT_TRY(staging().take((std::uint64_t)R * N * isz, &b.p));
+        const std::uint64_t st[4] = {(std::uint64_t)R * N * isz, (std::uint64_t)R * N * isz, (std::uint64_t)N * isz, isz};
+        TT_TRY(unpack_from(*qb, 0, 1, 0, 1, act_fmt, st, b.p, stream));
         bias_dev = b.p;  // row 0 of the tile-padded bias tensor
     }
-    // scratch for the forms that use it: W converted once into a bf16 panel (many rows), or partial sums of a split over K
-    // (shapes with few macro tiles)
-    Staged panel;
-    const std::uint64_t panel_bytes = ttbfp_gemm_bfp8b_workspace_bytes(M, N, K);
-    if (panel_bytes) TT_TRY(staging().take(panel_bytes, &panel.p));
-    TT_TRY(from_abi(ttbfp_gemm_bfp8b_bf16_ws(M, N, K, x.p, qw->base, bias_dev, epilogue, y.p,
-                                             TTBFP_FMT_FLOAT16_B, panel.p, panel_bytes, stream)));
-    {
-        std::unique_lock<std::mutex> l(qo->m);
-        if (qo->desc.io_type == IO_TYPE::Queue &&
-            !wait_until(l, qo->cv, timeout_s, [&] { return qo->count < qo->slots; }))
-            return fail("run_matmul: timed out waiting for space in " + out, DEVICE_STATUS_CODE::TimeoutError);
-        const std::uint32_t slot = qo->desc.io_type == IO_TYPE::Queue ? qo->wr : 0;
-        const std::uint64_t st[4] = {(std::uint64_t)M * N * 2, (std::uint64_t)M * N * 2, (std::uint64_t)N * 2, 2};
-        TT_TRY(pack_into(*qo, slot, (const std::uint8_t *)y.p, DataFormat::Float16_b, 1, st, stream));
-        TT_TRY(from_abi(ttbfp_stream_synchronize(stream, timeout_s)));
-        if (qo->desc.io_type == IO_TYPE::Queue) {
-            qo->wr = (qo->wr + 1) % qo->slots;
-            qo->count += 1;
-        }
-        qo->cv.notify_all();
+    if (full) {
+        TT_TRY(staging().take((std::uint64_t)K * N * 4, &w_full.p));
+        const std::uint64_t st[4] = {(std::uint64_t)K * N * 4, (std::uint64_t)K * N * 4, (std::uint64_t)N * 4, 4};
+        TT_TRY(unpack_from(*qw, 0, 1, 0, 1, DataFormat::Float32, st, w_full.p, stream));
+        TT_TRY(from_abi(ttbfp_gemm_f32(M, N, K, x.p, w_full.p, bias_dev, epilogue, y.p, stream)));
+    } else {
+        // scratch for the forms that use it: W converted once into a bf16 panel (many rows), or partial sums of a split over K
+        // (shapes with few macro tiles)
+        const std::uint64_t panel_bytes = ttbfp_gemm_bfp8b_workspace_bytes(M, N, K);
+        if (panel_bytes) TT_TRY(staging().take(panel_bytes, &panel.p));
+        TT_TRY(from_abi(ttbfp_gemm_bfp8b_bf16_ws(M, N, K, x.p, qw->base, bias_dev, epilogue, y.p,
+                                                 TTBFP_FMT_FLOAT16_B, panel.p, panel_bytes, stream)));
     }
+    Reservation r;
+    TT_TRY(reserve_write(*qo, 1, timeout_s, 0, r, "run_matmul"));
+    const std::uint64_t st[4] = {(std::uint64_t)M * N * isz, (std::uint64_t)M * N * isz, (std::uint64_t)N * isz, isz};
+    DEVICE_STATUS_CODE s = pack_into(*qo, r.slot0, (const std::uint8_t *)y.p, act_fmt, 1, st, stream);
+    if (s == DEVICE_STATUS_CODE::Success) s = sync_thread_stream(0);
+    publish_write(*qo, r, s == DEVICE_STATUS_CODE::Success);
+    TT_TRY(s);
     if (qa->desc.io_type == IO_TYPE::Queue) {
         std::lock_guard<std::mutex> l(qa->m);
         qa->rd = (qa->rd + 1) % qa->slots;
@@ -451,13 +700,16 @@ namespace backend {
 
 std::string last_error() { return g_last_error; }
 
+std::uint64_t pool_allocations() { return staging().allocations() + pinned().allocations(); }
+
 DEVICE_STATUS_CODE translate_addresses(tt_dram_io_desc &q)
 {
     return find_queue(q) ? DEVICE_STATUS_CODE::Success : fail("translate_addresses: unknown queue '" + q.queue_name + "'");
 }
 
 DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &qd, const tt_PytorchTensorDesc &t, const bool push_one,
-                              const int timeout_in_seconds, const int ram_ptr)
+                              const int timeout_in_seconds, const int ram_ptr, const bool tile_broadcast_r,
+                              const bool tile_broadcast_c)
 {
     auto q = find_queue(qd);
     if (!q) return fail("push_input: unknown queue '" + qd.queue_name + "'");
@@ -470,6 +722,10 @@ DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &qd, const tt_PytorchTensorD
     const bool prestride = ps > 0 && !qd.s_descriptor.xy_offsets.empty();
     std::uint32_t ps_rows_cols[2] = {0, 0};
     std::uint64_t ps_bytes = 0;
+    // Rows and columns that are not multiples of 32 are padded to the entry's tiles inside the pack launch: zeros, or for a
+    // dimension of one that is broadcast to its tile, copies of it (pad_pytorch_tensor_to_buda, pybuda/pybuda/tensor.py:805-877;
+    // pad_to_buda_shape, pybuda/csrc/tt_torch_device/tt_device.cpp:153-189).
+    std::uint32_t rows = 0, cols = 0;
     if (prestride) {
         if (qd.s_descriptor.xy_offsets.size() != (std::size_t)ps * ps) return fail("push_input: stride descriptor needs stride*stride offsets");
         for (int k = 0; k < ps * ps; ++k)
@@ -481,47 +737,47 @@ DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &qd, const tt_PytorchTensorD
             return fail("push_input: prestrided tensor [1," + std::to_string(ps_rows_cols[0]) + "," + std::to_string(ps_rows_cols[1]) +
                         "] does not match queue entry [t=" + std::to_string(d.t) + "," + std::to_string(d.rows()) + "," +
                         std::to_string(d.cols()) + "]");
-    } else if (t.shape[1] != d.t || t.shape[2] != d.rows() || t.shape[3] != d.cols())
-        return fail("push_input: tensor [" + std::to_string(t.shape[0]) + "," + std::to_string(t.shape[1]) + "," +
-                    std::to_string(t.shape[2]) + "," + std::to_string(t.shape[3]) + "] does not match queue entry [t=" +
-                    std::to_string(d.t) + "," + std::to_string(d.rows()) + "," + std::to_string(d.cols()) + "]");
+    } else {
+        if (t.shape[1] != d.t || align_up_tile(t.shape[2]) != d.rows() || align_up_tile(t.shape[3]) != d.cols())
+            return fail("push_input: tensor [" + std::to_string(t.shape[0]) + "," + std::to_string(t.shape[1]) + "," +
+                        std::to_string(t.shape[2]) + "," + std::to_string(t.shape[3]) + "] does not match queue entry [t=" +
+                        std::to_string(d.t) + "," + std::to_string(d.rows()) + "," + std::to_string(d.cols()) + "]");
+        rows = t.shape[2], cols = t.shape[3];
+        if ((tile_broadcast_r && rows != 1) || (tile_broadcast_c && cols != 1))
+            return fail("push_input: Trying to broadcast to tile dim a dimension that's not 1");
+    }
     const std::uint32_t n = t.shape[0];
     if (push_one && n != 1) return fail("push_input: push_one with " + std::to_string(n) + " entries in the tensor");
     if (n > q->slots) return fail("push_input: tensor holds more entries than the queue has slots");
 
-    std::unique_lock<std::mutex> l(q->m);
-    std::uint32_t slot0;
-    if (d.io_type == IO_TYPE::Queue) {
-        if (!wait_until(l, q->cv, timeout_in_seconds, [&] { return q->slots - q->count >= n; }))
-            return fail("push_input: queue '" + d.queue_name + "' is full", DEVICE_STATUS_CODE::TimeoutError);
-        slot0 = q->wr;
-    } else {
-        slot0 = ram_ptr < 0 ? 0 : (std::uint32_t)ram_ptr;
-        if (slot0 + n > q->slots) return fail("push_input: ram pointer past the end of '" + d.queue_name + "'");
-    }
-    void *stream = thread_stream();
-    Staged staged;
-    const std::uint8_t *dev_src = nullptr;
-    TT_TRY(stage_source(t, staged, &dev_src, stream));
-    const std::uint32_t first = std::min(n, q->slots - slot0);  // entries before the ring wraps
-    std::uint64_t st[4] = {t.strides[0], t.strides[1], t.strides[2], t.strides[3]};
-    Staged rearranged;
-    if (prestride) {
-        const std::uint32_t shape[4] = {t.shape[0], t.shape[1], t.shape[2], t.shape[3]};
-        TT_TRY(staging().take(ps_bytes, &rearranged.p));
-        TT_TRY(from_abi(ttbfp_prestride(dev_src, t.itemsize, shape, st, (std::uint32_t)ps, rearranged.p, ps_bytes, stream)));
-        dev_src = (const std::uint8_t *)rearranged.p;
-        st[3] = t.itemsize, st[2] = st[3] * ps_rows_cols[1], st[1] = st[2] * ps_rows_cols[0], st[0] = st[1];
-    }
-    TT_TRY(pack_into(*q, slot0, dev_src, t.format, first, st, stream));
-    if (first < n) TT_TRY(pack_into(*q, 0, dev_src + (std::uint64_t)first * st[0], t.format, n - first, st, stream));
-    TT_TRY(from_abi(ttbfp_stream_synchronize(stream, timeout_in_seconds)));
-    if (d.io_type == IO_TYPE::Queue) {
-        q->wr = (q->wr + n) % q->slots;
-        q->count += n;
-    }
-    q->cv.notify_all();
-    return DEVICE_STATUS_CODE::Success;
+    Reservation r;
+    TT_TRY(reserve_write(*q, n, timeout_in_seconds, ram_ptr, r, "push_input"));
+    // from here on the slots are ours: convert into them without the queue's lock, then publish
+    auto work = [&]() -> DEVICE_STATUS_CODE {
+        void *stream = thread_stream();
+        Staged staged, rearranged;
+        const std::uint8_t *dev_src = nullptr;
+        TT_TRY(stage_source(t, staged, &dev_src, stream));
+        const std::uint32_t first = std::min(n, q->slots - r.slot0);  // entries before the ring wraps
+        std::uint64_t st[4] = {t.strides[0], t.strides[1], t.strides[2], t.strides[3]};
+        if (prestride) {
+            const std::uint32_t shape[4] = {t.shape[0], t.shape[1], t.shape[2], t.shape[3]};
+            TT_TRY(staging().take(ps_bytes, &rearranged.p));
+            TT_TRY(from_abi(ttbfp_prestride(dev_src, t.itemsize, shape, st, (std::uint32_t)ps, rearranged.p, ps_bytes, stream)));
+            dev_src = (const std::uint8_t *)rearranged.p;
+            st[3] = t.itemsize, st[2] = st[3] * ps_rows_cols[1], st[1] = st[2] * ps_rows_cols[0], st[0] = st[1];
+        }
+        TT_TRY(pack_into(*q, r.slot0, dev_src, t.format, first, st, stream, rows, cols, tile_broadcast_r, tile_broadcast_c));
+        if (first < n)
+            TT_TRY(pack_into(*q, 0, dev_src + (std::uint64_t)first * st[0], t.format, n - first, st, stream, rows, cols, tile_broadcast_r,
+                             tile_broadcast_c));
+        // the time limit of this call is for space in the queue (as in the reference, whose pushes time out on a full
+        // queue); the conversion itself is bounded work and is always waited for
+        return sync_thread_stream(0);
+    };
+    const DEVICE_STATUS_CODE s = work();
+    publish_write(*q, r, s == DEVICE_STATUS_CODE::Success);
+    return s;
 }
 
 DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &qd, const tt_TilizedTensorDesc &t, const int timeout_in_seconds,
@@ -529,9 +785,10 @@ DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &qd, const tt_TilizedTensorD
 {
     auto q = find_queue(qd);
     if (!q) return fail("push_input: unknown queue '" + qd.queue_name + "'");
-    const tt_dram_io_desc &d = q->desc;
     if (!t.ptr) return fail("push_input: tilized descriptor has no data (load it with debinarize_tensor)");
-    if (t.format != d.bufq_target_format) return fail("push_input: tilized tensor format differs from the queue format");
+    if (t.format != q->storage)
+        return fail(std::string("push_input: tilized tensor format ") + data_format_name(t.format) + " differs from the format the queue holds, " +
+                    data_format_name(q->storage));
     if (t.num_buffers != q->buffers)
         return fail("push_input: tilized tensor has " + std::to_string(t.num_buffers) + " buffers, the queue's grid has " +
                     std::to_string(q->buffers));
@@ -540,36 +797,30 @@ DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &qd, const tt_TilizedTensorD
     const std::uint32_t n = (std::uint32_t)(t.buf_size_bytes / q->entry_bytes);
     if (n > q->slots) return fail("push_input: tensor holds more entries than the queue has slots");
 
-    std::unique_lock<std::mutex> l(q->m);
-    std::uint32_t slot0;
-    if (d.io_type == IO_TYPE::Queue) {
-        if (!wait_until(l, q->cv, timeout_in_seconds, [&] { return q->slots - q->count >= n; }))
-            return fail("push_input: queue '" + d.queue_name + "' is full", DEVICE_STATUS_CODE::TimeoutError);
-        slot0 = q->wr;
-    } else {
-        slot0 = ram_ptr < 0 ? 0 : (std::uint32_t)ram_ptr;
-        if (slot0 + n > q->slots) return fail("push_input: ram pointer past the end of '" + d.queue_name + "'");
-    }
-    void *stream = thread_stream();
-    const bool on_device = ttbfp_pointer_is_device(t.ptr);
-    auto copy = on_device ? ttbfp_memcpy_d2d : ttbfp_memcpy_h2d;
-    const std::uint32_t first = std::min(n, q->slots - slot0);
-    for (std::uint32_t b = 0; b < q->buffers; ++b) {  // buffer b of the tensor into buffer b of the queue
-        const std::uint8_t *from = (const std::uint8_t *)t.ptr + (std::uint64_t)b * t.buf_size_bytes;
-        TT_TRY(from_abi(copy(q->slot(slot0) + b * q->pitch, from, first * q->entry_bytes, stream)));
-        if (first < n) TT_TRY(from_abi(copy(q->base + b * q->pitch, from + first * q->entry_bytes, (n - first) * q->entry_bytes, stream)));
-    }
-    TT_TRY(from_abi(ttbfp_stream_synchronize(stream, timeout_in_seconds)));
-    if (d.io_type == IO_TYPE::Queue) {
-        q->wr = (q->wr + n) % q->slots;
-        q->count += n;
-    }
-    q->cv.notify_all();
-    return DEVICE_STATUS_CODE::Success;
+    Reservation r;
+    TT_TRY(reserve_write(*q, n, timeout_in_seconds, ram_ptr, r, "push_input"));
+    auto work = [&]() -> DEVICE_STATUS_CODE {
+        void *stream = thread_stream();
+        const bool on_device = ttbfp_pointer_is_device(t.ptr);
+        if (on_device) TT_TRY(from_abi(ttbfp_device_synchronize()));  // the producer's stream is not known here
+        auto copy = on_device ? ttbfp_memcpy_d2d : ttbfp_memcpy_h2d;
+        const std::uint32_t first = std::min(n, q->slots - r.slot0);
+        for (std::uint32_t b = 0; b < q->buffers; ++b) {  // buffer b of the tensor into buffer b of the queue
+            const std::uint8_t *from = (const std::uint8_t *)t.ptr + (std::uint64_t)b * t.buf_size_bytes;
+            TT_TRY(from_abi(copy(q->slot(r.slot0) + b * q->pitch, from, first * q->entry_bytes, stream)));
+            if (first < n) TT_TRY(from_abi(copy(q->base + b * q->pitch, from + first * q->entry_bytes, (n - first) * q->entry_bytes, stream)));
+        }
+        return sync_thread_stream(0);
+    };
+    const DEVICE_STATUS_CODE s = work();
+    if (s != DEVICE_STATUS_CODE::Success) drain_thread_stream();  // the caller's memory must not be read after the call returns
+    publish_write(*q, r, s == DEVICE_STATUS_CODE::Success);
+    return s;
 }
 
 DEVICE_STATUS_CODE get_output(const tt_dram_io_desc &qd, tt_PytorchTensorDesc &out, const bool pop_one,
-                              const int timeout_in_seconds, const int rd_ptr)
+                              const int timeout_in_seconds, const int rd_ptr, const std::uint32_t narrow_r,
+                              const std::uint32_t narrow_c)
 {
     auto q = find_queue(qd);
     if (!q) return fail("get_output: unknown queue '" + qd.queue_name + "'");
@@ -582,62 +833,66 @@ DEVICE_STATUS_CODE get_output(const tt_dram_io_desc &qd, tt_PytorchTensorDesc &o
     if (d.t % (hs * vs) != 0) return fail("get_output: t is not divisible by hstack_factor * vstack_factor");
     const std::uint32_t n = pop_one ? 1 : d.input_count;
     if (n > q->slots) return fail("get_output: input_count exceeds the queue's slots");
+    // narrow_r / narrow_c (0: keep all): only that many rows / columns of every slice are unpacked and copied back, the
+    // narrowing of narrow_buda_tensor_to_pytorch (pybuda/pybuda/tensor.py:879-954) done inside the launch
+    const std::uint32_t R = narrow_r ? narrow_r : d.rows(), C = narrow_c ? narrow_c : d.cols();
+    if (R > d.rows() || C > d.cols() || align_up_tile(R) != d.rows() || align_up_tile(C) != d.cols())
+        return fail("get_output: cannot narrow an entry of " + std::to_string(d.rows()) + " x " + std::to_string(d.cols()) + " to " +
+                    std::to_string(R) + " x " + std::to_string(C) + " (the tiles must be those of the narrowed shape)");
+    const bool narrowed = R != d.rows() || C != d.cols();
+    if (narrowed && (hs != 1 || vs != 1)) return fail("get_output: narrowing does not combine with hstack / vstack");
 
-    std::unique_lock<std::mutex> l(q->m);
-    std::uint32_t slot0;
-    if (d.io_type == IO_TYPE::Queue) {
-        if (!wait_until(l, q->cv, timeout_in_seconds, [&] { return q->count >= n; }))
-            return fail("get_output: queue '" + d.queue_name + "' is empty", DEVICE_STATUS_CODE::TimeoutError);
-        slot0 = rd_ptr >= 0 ? (std::uint32_t)rd_ptr % q->slots : q->rd;
-    } else {
-        slot0 = rd_ptr < 0 ? 0 : (std::uint32_t)rd_ptr;
-        if (slot0 + n > q->slots) return fail("get_output: read pointer past the end of '" + d.queue_name + "'");
-    }
     // Output formats are the ones pybuda turns back into torch tensors (pybuda/pybuda/tensor.py:730-740):
     // Float32 queues read back as Float32, everything with an 8-bit exponent as Float16_b, unless the
     // caller asked for Float32 by presetting the descriptor's format.
-    DataFormat of = d.bufq_target_format == DataFormat::RawUInt32 ? DataFormat::RawUInt32
-                    : a_family(d.bufq_target_format)             ? DataFormat::Float16
-                    : out.format == DataFormat::Float32            ? DataFormat::Float32
-                    : d.bufq_target_format == DataFormat::Float32 ? DataFormat::Float32
-                                                                  : DataFormat::Float16_b;
+    DataFormat of = q->storage == DataFormat::RawUInt32 ? DataFormat::RawUInt32
+                    : a_family(q->storage)              ? DataFormat::Float16
+                    : out.format == DataFormat::Float32 ? DataFormat::Float32
+                    : q->storage == DataFormat::Float32 ? DataFormat::Float32
+                                                        : DataFormat::Float16_b;
     const std::uint32_t isz = data_format_byte_size(of);
-    const std::uint32_t R = d.rows(), C = d.cols();
     const std::uint64_t per_entry = (std::uint64_t)d.t * R * C * isz;
     if (per_entry * n > 0xffffffffull) return fail("get_output: result exceeds the 32-bit strides of the descriptor");
-    void *stream = thread_stream();
-    Staged dev;
-    TT_TRY(staging().take(per_entry * n, &dev.p));
+
+    std::uint32_t slot0 = 0;
+    TT_TRY(begin_read(*q, n, timeout_in_seconds, rd_ptr, slot0, "get_output"));
+    void *host = nullptr;
     // result [n, t/(h v), R v, C h]: row pitch C h, slice pitch R v rows
     const std::uint64_t row_pitch = (std::uint64_t)C * hs * isz, slice_pitch = (std::uint64_t)R * vs * row_pitch;
     const std::uint64_t st[4] = {per_entry, slice_pitch, row_pitch, isz};
-    const std::uint32_t first = std::min(n, q->slots - slot0);
-    auto unpack_range = [&](std::uint32_t slot, std::uint32_t entries, std::uint8_t *dst) -> DEVICE_STATUS_CODE {
-        if (hs == 1 && vs == 1) return unpack_from(*q, slot, entries, 0, d.t, of, st, dst, stream);
-        // one launch per run of z slices that land at a constant pitch: the fastest index of the group
-        const bool h_fast = qd.stack_row_major != 0 || vs == 1;
-        const std::uint32_t run = h_fast ? hs : vs, outer = h_fast ? vs : hs;
-        const std::uint64_t run_pitch = h_fast ? (std::uint64_t)C * isz : (std::uint64_t)R * row_pitch;
-        const std::uint64_t outer_pitch = h_fast ? (std::uint64_t)R * row_pitch : (std::uint64_t)C * isz;
-        const std::uint64_t run_st[4] = {0, run_pitch, row_pitch, isz};
-        for (std::uint32_t e = 0; e < entries; ++e)
-            for (std::uint32_t zo = 0; zo < d.t / (hs * vs); ++zo)
-                for (std::uint32_t o = 0; o < outer; ++o) {
-                    const std::uint32_t z0 = (zo * outer + o) * run;
-                    DEVICE_STATUS_CODE s = unpack_from(*q, slot + e, 1, z0, run, of, run_st,
-                                                       dst + e * per_entry + zo * slice_pitch + o * outer_pitch, stream);
-                    if (s != DEVICE_STATUS_CODE::Success) return s;
-                }
-        return DEVICE_STATUS_CODE::Success;
+    auto work = [&]() -> DEVICE_STATUS_CODE {
+        void *stream = thread_stream();
+        Staged dev;
+        TT_TRY(staging().take(per_entry * n, &dev.p));
+        const std::uint32_t first = std::min(n, q->slots - slot0);
+        auto unpack_range = [&](std::uint32_t slot, std::uint32_t entries, std::uint8_t *dst) -> DEVICE_STATUS_CODE {
+            if (hs == 1 && vs == 1) return unpack_from(*q, slot, entries, 0, d.t, of, st, dst, stream, R, C);
+            // one launch per run of z slices that land at a constant pitch: the fastest index of the group
+            const bool h_fast = qd.stack_row_major != 0 || vs == 1;
+            const std::uint32_t run = h_fast ? hs : vs, outer = h_fast ? vs : hs;
+            const std::uint64_t run_pitch = h_fast ? (std::uint64_t)C * isz : (std::uint64_t)R * row_pitch;
+            const std::uint64_t outer_pitch = h_fast ? (std::uint64_t)R * row_pitch : (std::uint64_t)C * isz;
+            const std::uint64_t run_st[4] = {0, run_pitch, row_pitch, isz};
+            for (std::uint32_t e = 0; e < entries; ++e)
+                for (std::uint32_t zo = 0; zo < d.t / (hs * vs); ++zo)
+                    for (std::uint32_t o = 0; o < outer; ++o) {
+                        const std::uint32_t z0 = (zo * outer + o) * run;
+                        DEVICE_STATUS_CODE s = unpack_from(*q, slot + e, 1, z0, run, of, run_st,
+                                                           dst + e * per_entry + zo * slice_pitch + o * outer_pitch, stream);
+                        if (s != DEVICE_STATUS_CODE::Success) return s;
+                    }
+            return DEVICE_STATUS_CODE::Success;
+        };
+        TT_TRY(unpack_range(slot0, first, (std::uint8_t *)dev.p));
+        if (first < n) TT_TRY(unpack_range(0, n - first, (std::uint8_t *)dev.p + first * per_entry));
+        TT_TRY(host_block(per_entry * n, &host));
+        TT_TRY(from_abi(ttbfp_memcpy_d2h(host, dev.p, per_entry * n, stream)));
+        return sync_thread_stream(0);  // the time limit is for entries to arrive; reading them is bounded work
     };
-    TT_TRY(unpack_range(slot0, first, (std::uint8_t *)dev.p));
-    if (first < n) TT_TRY(unpack_range(0, n - first, (std::uint8_t *)dev.p + first * per_entry));
-    void *host = nullptr;
-    TT_TRY(host_block(per_entry * n, &host));
-    DEVICE_STATUS_CODE s = from_abi(ttbfp_memcpy_d2h(host, dev.p, per_entry * n, stream));
-    if (s == DEVICE_STATUS_CODE::Success) s = from_abi(ttbfp_stream_synchronize(stream, timeout_in_seconds));
+    const DEVICE_STATUS_CODE s = work();
+    end_read(*q);
     if (s != DEVICE_STATUS_CODE::Success) {
-        release_host_block(host);
+        if (host) release_host_block(host);
         return s;
     }
     out.ptr = host;
@@ -655,14 +910,7 @@ DEVICE_STATUS_CODE pop_output(const tt_dram_io_desc &qd, const bool pop_one, con
     auto q = find_queue(qd);
     if (!q) return fail("pop_output: unknown queue '" + qd.queue_name + "'");
     if (q->desc.io_type != IO_TYPE::Queue) return DEVICE_STATUS_CODE::Success;  // nothing to release in a RAM
-    const std::uint32_t n = pop_one ? 1 : q->desc.input_count;
-    std::unique_lock<std::mutex> l(q->m);
-    if (!wait_until(l, q->cv, timeout_in_seconds, [&] { return q->count >= n; }))
-        return fail("pop_output: queue '" + q->desc.queue_name + "' is empty", DEVICE_STATUS_CODE::TimeoutError);
-    q->rd = (q->rd + n) % q->slots;
-    q->count -= n;
-    q->cv.notify_all();
-    return DEVICE_STATUS_CODE::Success;
+    return release_entries(*q, pop_one ? 1 : q->desc.input_count, timeout_in_seconds, "pop_output");
 }
 
 template <>
@@ -687,8 +935,11 @@ tt_TilizedTensorDesc tilize_tensor(const tt_dram_io_desc &qd, const tt_PytorchTe
     auto must = [](DEVICE_STATUS_CODE s) {
         if (s != DEVICE_STATUS_CODE::Success) throw std::runtime_error("tilize_tensor: " + g_last_error);
     };
-    const DataFormat fmt = qd.bufq_target_format;
-    must(check_source(t, fmt, "tilize_tensor"));
+    // the descriptor of a registered queue tilizes into the format that queue holds (its declared format, or the
+    // full-precision stand-in of a backend that ignores data-format precision); any other descriptor into the one it names
+    const auto registered = find_queue(qd);
+    const DataFormat fmt = registered ? registered->storage : qd.bufq_target_format;
+    must(check_source(t, qd.bufq_target_format, "tilize_tensor"));
     const std::uint32_t shape[4] = {t.shape[0], t.shape[1], t.shape[2], t.shape[3]};
     if (ttbfp_packed_size((std::uint8_t)fmt, shape) == 0)
         must(fail("rows and columns must be multiples of 32 (pad with pad_pytorch_tensor_to_buda first)"));
@@ -705,22 +956,56 @@ tt_TilizedTensorDesc tilize_tensor(const tt_dram_io_desc &qd, const tt_PytorchTe
     const std::uint64_t per_buffer = ttbfp_queue_buffer_bytes((std::uint8_t)fmt, shape, &lay), bytes = per_buffer * buffers;
     if (per_buffer == 0 || per_buffer > 0xffffffffull) must(fail("tilized size does not fit the descriptor (one buffer is limited to 4 GiB)"));
     void *stream = thread_stream();
-    Staged src, dst;
-    const std::uint8_t *dev_src = nullptr;
-    must(stage_source(t, src, &dev_src, stream));
-    must(staging().take(bytes, &dst.p));
-    const std::uint64_t st[4] = {t.strides[0], t.strides[1], t.strides[2], t.strides[3]};
-    must(from_abi(ttbfp_tilize_pack_queue(dev_src, (std::uint8_t)t.format, shape, st, (std::uint8_t)fmt, conversion_rounding(), &lay,
-                                          per_buffer, dst.p, bytes, stream)));
     void *host = nullptr;
-    must(host_block(bytes, &host));
-    DEVICE_STATUS_CODE s = from_abi(ttbfp_memcpy_d2h(host, dst.p, bytes, stream));
-    if (s == DEVICE_STATUS_CODE::Success) s = from_abi(ttbfp_stream_synchronize(stream, 0));
-    if (s != DEVICE_STATUS_CODE::Success) {
-        release_host_block(host);
-        must(s);
+    try {
+        Staged src, dst;
+        const std::uint8_t *dev_src = nullptr;
+        must(stage_source(t, src, &dev_src, stream));
+        must(staging().take(bytes, &dst.p));
+        const std::uint64_t st[4] = {t.strides[0], t.strides[1], t.strides[2], t.strides[3]};
+        must(from_abi(ttbfp_tilize_pack_queue(dev_src, (std::uint8_t)t.format, shape, st, (std::uint8_t)fmt, conversion_rounding(), &lay,
+                                              per_buffer, dst.p, bytes, stream)));
+        must(host_block(bytes, &host));
+        must(from_abi(ttbfp_memcpy_d2h(host, dst.p, bytes, stream)));
+        must(sync_thread_stream(0));
+    } catch (...) {
+        if (host) release_host_block(host);  // drains the stream first
+        throw;
     }
     return tt_TilizedTensorDesc(host, buffers, (std::uint32_t)per_buffer, fmt);
+}
+
+// The C++ caller's padding (pybuda/csrc/tt_torch_device/tt_device.cpp:153-189): a tensor of up to four dimensions becomes
+// 4-D (leading ones), its rows and columns are rounded up to whole tiles (align_up_tile, tt_device.hpp:205-210) and filled
+// with zeros, and the result is contiguous.  The result lives in backend-owned pinned memory (free_tensor releases it).
+// push_input does not need this step - it pads inside its pack launch - so this is for callers that want the padded
+// tensor itself.
+tt_PytorchTensorDesc pad_to_buda_shape(const tt_PytorchTensorDesc &t)
+{
+    if (!t.ptr) throw std::runtime_error("pad_to_buda_shape: tensor descriptor has no data pointer");
+    if (ttbfp_pointer_is_device(t.ptr)) throw std::runtime_error("pad_to_buda_shape: the tensor must be in host memory");
+    if (t.itemsize == 0 || t.itemsize > 8) throw std::runtime_error("pad_to_buda_shape: bad itemsize");
+    const std::uint32_t R = align_up_tile(t.shape[2]), C = align_up_tile(t.shape[3]);
+    const std::uint64_t row = (std::uint64_t)C * t.itemsize, slice = row * R, bytes = slice * t.shape[0] * t.shape[1];
+    if (bytes > 0xffffffffull) throw std::runtime_error("pad_to_buda_shape: result exceeds the 32-bit strides of the descriptor");
+    void *host = nullptr;
+    if (host_block(bytes, &host) != DEVICE_STATUS_CODE::Success) throw std::runtime_error("pad_to_buda_shape: " + g_last_error);
+    std::memset(host, 0, bytes);
+    for (std::uint32_t w = 0; w < t.shape[0]; ++w)
+        for (std::uint32_t z = 0; z < t.shape[1]; ++z)
+            for (std::uint32_t r = 0; r < t.shape[2]; ++r) {
+                const std::uint8_t *src = (const std::uint8_t *)t.ptr + (std::uint64_t)w * t.strides[0] + (std::uint64_t)z * t.strides[1] +
+                                          (std::uint64_t)r * t.strides[2];
+                std::uint8_t *dst = (std::uint8_t *)host + ((std::uint64_t)w * t.shape[1] + z) * slice + r * row;
+                if (t.strides[3] == t.itemsize) {
+                    std::memcpy(dst, src, (std::size_t)t.shape[3] * t.itemsize);
+                } else {
+                    for (std::uint32_t c = 0; c < t.shape[3]; ++c)
+                        std::memcpy(dst + (std::size_t)c * t.itemsize, src + (std::uint64_t)c * t.strides[3], t.itemsize);
+                }
+            }
+    return tt_PytorchTensorDesc(host, t.itemsize, t.format, {t.shape[0], t.shape[1], R, C},
+                                {(std::uint32_t)(slice * t.shape[1]), (std::uint32_t)slice, (std::uint32_t)row, t.itemsize}, 4);
 }
 
 namespace {

@@ -21,6 +21,35 @@ enum class IO_TYPE : int { Queue = 0, RandomAccess = 1, Invalid = 0xff };
 enum class IO_LAYOUT : int { Tilized = 0, Flat = 1, Invalid = 0xff };
 // The only device kind this backend drives.
 enum class DEVICE : int { Hip = 0, Invalid = 0xff };
+// The part it drives, and how a backend object is used (the reference's BackendDevice and DeviceMode arguments of
+// BackendConfig, pybuda/csrc/backend_api/backend_api.cpp:243-260); kept so that the constructor takes the same arguments.
+enum class ARCH : int { MI355X = 0, Invalid = 0xff };
+enum class DEVICE_MODE : int { CompileAndRun = 0, CompileOnly = 1, RunOnly = 2 };
+
+// pybuda/csrc/tt_torch_device/tt_device.hpp:205-210
+template <typename T>
+inline T align_up_tile(T d)
+{
+    return static_cast<T>((d + 31) / 32 * 32);
+}
+
+// tt_backend_config as far as this backend reads it (backend_api.cpp:243-281).  ignore_data_format_precision is the
+// golden-precision switch: false (the default of a device backend) keeps every queue in its declared DataFormat, so
+// tensors are quantized on the way in and the matmul runs on the dequantized values; true ("run backend at full precision",
+// what the reference's Golden device does unless told otherwise, backend_api.cpp:268-270, pybuda/pybuda/verify/config.py:67)
+// keeps queues unquantized and evaluates in fp32.
+struct tt_backend_config {
+    DEVICE type = DEVICE::Hip;
+    ARCH arch = ARCH::MI355X;
+    DEVICE_MODE mode = DEVICE_MODE::CompileAndRun;
+    int optimization_level = 0;
+    std::string output_dir;
+    std::string soc_descriptor_path;
+    std::string cluster_descriptor_path;
+    bool ignore_data_format_precision = false;
+    std::string perf_desc_args;
+    std::string runtime_args;
+};
 
 // backend_api.cpp:384-407
 struct Stride {
@@ -103,7 +132,7 @@ int conversion_rounding();
 // from a netlist; here they are declared one by one with create_queue.
 class tt_backend {
    public:
-    static std::shared_ptr<tt_backend> create(int device = 0);
+    static std::shared_ptr<tt_backend> create(int device = 0, const tt_backend_config &config = tt_backend_config());
     ~tt_backend();
 
     DEVICE_STATUS_CODE initialize();
@@ -120,11 +149,18 @@ class tt_backend {
                                  std::uint32_t input_count = 1, std::uint32_t grid_r = 1, std::uint32_t grid_c = 1,
                                  std::uint32_t ublock_order = 0, bool tile_header = false);
     tt_dram_io_desc get_queue_descriptor(const std::string &name) const;
+    // The format of the tiles a queue holds in HBM: its declared format, or with ignore_data_format_precision the
+    // full-precision stand-in (Float32 for the formats with an 8-bit exponent, Float16 for those with five).
+    DataFormat queue_storage_format(const std::string &name) const;
+    // The largest number of push_input / get_output / run_matmul conversions that ever ran on this queue at one time.
+    std::uint32_t queue_max_in_flight(const std::string &name) const;
+    const tt_backend_config &config() const { return config_; }
 
     // out = epilogue(in0 * weight + bias): the matmul op of a netlist program, evaluated with the
     // Bfp8_b-weight GEMM.  in0 and out are Float16_b queues, weight a Bfp8_b RandomAccess queue
     // holding W[K,N], bias (optional, "" = none) a Float16_b RandomAccess queue whose row 0 is
-    // broadcast (pybuda/pybuda/op/eval/buda/matmul.py:233-249).  Consumes one entry of in0 and
+    // broadcast (pybuda/pybuda/op/eval/buda/matmul.py:233-249).  With ignore_data_format_precision the queues hold
+    // unquantized fp32 tiles whatever their declared formats, and the product is an fp32 matmul on them.  Consumes one entry of in0 and
     // produces one entry of out.  gelu: apply GELU to the result, in the form `approximate` names ("none": erf form,
     // "tanh": pybuda/pybuda/op/eval/pybuda/eltwise_unary.py:42-49; anything else is an error as it is there).
     DEVICE_STATUS_CODE run_matmul(const std::string &in0, const std::string &weight, const std::string &bias,
@@ -133,20 +169,28 @@ class tt_backend {
     const std::string &id() const { return id_; }
 
    private:
-    explicit tt_backend(int device);
+    tt_backend(int device, const tt_backend_config &config);
     int device_;
+    tt_backend_config config_;
     std::string id_;
     std::vector<std::string> queues_;
 };
 
 namespace backend {
 
+// Rows and columns of the tensor that are not multiples of 32 are padded to the entry's tiles inside the pack launch
+// (zeros; with tile_broadcast_r / tile_broadcast_c a dimension of one is copied through its tile instead, the "replicate"
+// mode of pad_pytorch_tensor_to_buda, pybuda/pybuda/tensor.py:848-856).  timeout_in_seconds bounds the wait for free slots.
 DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &q, const tt_PytorchTensorDesc &tensor, const bool push_one,
-                              const int timeout_in_seconds, const int ram_ptr);
+                              const int timeout_in_seconds, const int ram_ptr, const bool tile_broadcast_r = false,
+                              const bool tile_broadcast_c = false);
 DEVICE_STATUS_CODE push_input(const tt_dram_io_desc &q, const tt_TilizedTensorDesc &tensor, const int timeout_in_seconds,
                               const int ram_ptr);
+// narrow_r / narrow_c (0: the whole entry): the result keeps only that many rows / columns of every slice
+// (narrow_buda_tensor_to_pytorch, pybuda/pybuda/tensor.py:879-954, inside the unpack launch).
 DEVICE_STATUS_CODE get_output(const tt_dram_io_desc &q, tt_PytorchTensorDesc &out, const bool pop_one,
-                              const int timeout_in_seconds, const int rd_ptr);
+                              const int timeout_in_seconds, const int rd_ptr, const std::uint32_t narrow_r = 0,
+                              const std::uint32_t narrow_c = 0);
 DEVICE_STATUS_CODE pop_output(const tt_dram_io_desc &q, const bool pop_one, const int timeout_in_seconds);
 DEVICE_STATUS_CODE translate_addresses(tt_dram_io_desc &q);
 
@@ -156,6 +200,14 @@ DEVICE_STATUS_CODE free_tensor(T &desc);
 // Row-major host (or device) tensor -> tiles in the queue's format, in backend-owned pinned host
 // memory; release with free_tensor.  Throws std::runtime_error on failure, as the reference does.
 tt_TilizedTensorDesc tilize_tensor(const tt_dram_io_desc &q, const tt_PytorchTensorDesc &tensor);
+
+// Host tensor of up to four dimensions -> 4-D, rows and columns zero-padded to whole tiles, contiguous, in backend-owned
+// pinned memory (pybuda/csrc/tt_torch_device/tt_device.cpp:153-189).  Throws std::runtime_error on failure.
+tt_PytorchTensorDesc pad_to_buda_shape(const tt_PytorchTensorDesc &tensor);
+
+// Device and pinned-host blocks the pools behind push_input / get_output / tilize_tensor / run_matmul have allocated so far:
+// constant in steady state.
+std::uint64_t pool_allocations();
 
 template <typename T>
 void binarize_tensor(const T &desc, std::string file_path);

@@ -90,6 +90,40 @@ void bind_backend(py::module &m)
         .value("Invalid", IO_LAYOUT::Invalid);
 
     py::enum_<DEVICE>(m, "BackendType").value("Hip", DEVICE::Hip).value("NoBackend", DEVICE::Invalid);
+    py::enum_<ARCH>(m, "BackendDevice").value("MI355X", ARCH::MI355X).value("Invalid", ARCH::Invalid);
+    py::enum_<DEVICE_MODE>(m, "DeviceMode")
+        .value("CompileAndRun", DEVICE_MODE::CompileAndRun)
+        .value("CompileOnly", DEVICE_MODE::CompileOnly)
+        .value("RunOnly", DEVICE_MODE::RunOnly);
+
+    // Same constructor arguments and setters as the reference's BackendConfig (backend_api.cpp:243-281); the descriptor
+    // paths are kept and not read (there is no SoC or cluster description to load).
+    py::class_<tt_backend_config>(m, "BackendConfig")
+        .def(py::init([](DEVICE backend_type, ARCH backend_device, DEVICE_MODE device_mode, int opt_level, const std::string &output_dir,
+                         const std::string &soc_descriptor_path, const std::string &cluster_descriptor_path) {
+                 tt_backend_config cfg;
+                 cfg.type = backend_type;
+                 cfg.arch = backend_device;
+                 cfg.mode = device_mode;
+                 cfg.output_dir = output_dir;
+                 cfg.soc_descriptor_path = soc_descriptor_path;
+                 cfg.cluster_descriptor_path = cluster_descriptor_path;
+                 const char *env_opt_level = std::getenv("TT_BACKEND_OPT_LEVEL");
+                 cfg.optimization_level = env_opt_level ? std::atoi(env_opt_level) : opt_level;
+                 return cfg;
+             }),
+             py::arg("backend_type") = DEVICE::Hip, py::arg("backend_device") = ARCH::MI355X,
+             py::arg("device_mode") = DEVICE_MODE::CompileAndRun, py::arg("opt_level") = 0, py::arg("output_dir") = "",
+             py::arg("soc_descriptor_path") = "", py::arg("cluster_descriptor_path") = "")
+        .def("set_golden_ignore_df_precision",
+             [](tt_backend_config &self, bool ignore_data_format_precision) { self.ignore_data_format_precision = ignore_data_format_precision; })
+        .def("set_performance_trace_args", [](tt_backend_config &self, std::string args) { self.perf_desc_args = args; })
+        .def("set_runtime_args", [](tt_backend_config &self, std::string args) { self.runtime_args = args; })
+        .def_readonly("ignore_data_format_precision", &tt_backend_config::ignore_data_format_precision)
+        .def_readonly("optimization_level", &tt_backend_config::optimization_level)
+        .def_readonly("output_dir", &tt_backend_config::output_dir)
+        .def_readonly("perf_desc_args", &tt_backend_config::perf_desc_args)
+        .def_readonly("runtime_args", &tt_backend_config::runtime_args);
 
     py::class_<Stride>(m, "StrideDescriptor")
         .def(py::init<>())
@@ -246,7 +280,10 @@ void bind_backend(py::module &m)
                         }));
 
     py::class_<tt_backend, std::shared_ptr<tt_backend>>(m, "BackendApi")
-        .def(py::init(&tt_backend::create), py::arg("device") = 0)
+        .def(py::init(&tt_backend::create), py::arg("device") = 0, py::arg("config") = tt_backend_config())
+        .def("get_config", &tt_backend::config)
+        .def("queue_storage_format", &tt_backend::queue_storage_format)
+        .def("queue_max_in_flight", &tt_backend::queue_max_in_flight)
         .def("initialize", &tt_backend::initialize, py::call_guard<py::gil_scoped_release>())
         .def("finish", &tt_backend::finish)
         .def("wait_for_idle", &tt_backend::wait_for_idle, py::call_guard<py::gil_scoped_release>())
@@ -261,15 +298,21 @@ void bind_backend(py::module &m)
 
     m.def("release_backend_ptr", [](std::shared_ptr<tt_backend> b) { b.reset(); });
 
+    // the reference's five positional arguments, then the two tile-broadcast flags of this build
     m.def("push_input",
-          py::overload_cast<const tt_dram_io_desc &, const tt_PytorchTensorDesc &, const bool, const int, const int>(
+          py::overload_cast<const tt_dram_io_desc &, const tt_PytorchTensorDesc &, const bool, const int, const int, const bool, const bool>(
               &backend::push_input),
-          py::call_guard<py::gil_scoped_release>());
+          py::arg("queue"), py::arg("tensor"), py::arg("push_one"), py::arg("timeout"), py::arg("ram_ptr"),
+          py::arg("tile_broadcast_r") = false, py::arg("tile_broadcast_c") = false, py::call_guard<py::gil_scoped_release>());
     m.def("push_input",
           py::overload_cast<const tt_dram_io_desc &, const tt_TilizedTensorDesc &, const int, const int>(&backend::push_input),
           py::call_guard<py::gil_scoped_release>());
     m.def("pop_output", &backend::pop_output, py::call_guard<py::gil_scoped_release>());
-    m.def("get_output", &backend::get_output, py::call_guard<py::gil_scoped_release>());
+    m.def("get_output", &backend::get_output, py::arg("queue"), py::arg("out"), py::arg("pop_one"), py::arg("timeout"), py::arg("rd_ptr"),
+          py::arg("narrow_r") = 0, py::arg("narrow_c") = 0, py::call_guard<py::gil_scoped_release>());
+    m.def("pad_to_buda_shape", &backend::pad_to_buda_shape);
+    m.def("align_up_tile", [](std::uint32_t d) { return align_up_tile(d); });
+    m.def("pool_allocations", &backend::pool_allocations);
     m.def("free_tensor", &backend::free_tensor<tt_PytorchTensorDesc>);
     m.def("free_tensor", &backend::free_tensor<tt_TilizedTensorDesc>);
     m.def("tilize_tensor", &backend::tilize_tensor);

@@ -82,17 +82,11 @@ def matmul(x: torch.Tensor, w: BfpWeight, bias: Optional[torch.Tensor] = None, g
     xs = x.reshape(w.Z, M, w.K).to(device="cuda", dtype=torch.bfloat16)
     brow = _bias_row(bias, w.N)
     if accumulate:
-        # sum_z (x_z w_z + b) = [x_0 .. x_{Z-1}] [w_0; ..; w_{Z-1}] + Z b; the bias rides in the GEMM when Z b is a bf16 value
+        # sum_z (x_z w_z + b) = [x_0 .. x_{Z-1}] [w_0; ..; w_{Z-1}] + Z b; Z b is not a bf16 value in general, so it rides in the
+        # GEMM's epilogue as an fp32 bias
         x2 = xs.permute(1, 0, 2).reshape(M, w.Z * w.K).contiguous()
-        total = None if brow is None else brow.float() * w.Z
-        fused = total is None or bool(torch.equal(total.bfloat16().float(), total))
-        if fused:
-            y = capi.gemm_bfp8b(x2, w.packed, w.N, bias=None if total is None else total.bfloat16(), epilogue=epilogue, out_dtype=out_dtype)
-        else:
-            y = capi.gemm_bfp8b(x2, w.packed, w.N, out_dtype=torch.float32) + total
-            if epilogue != capi.EPILOGUE_NONE:
-                y = torch.nn.functional.gelu(y, approximate="tanh" if epilogue == capi.EPILOGUE_GELU_TANH else "none")
-            y = y.to(out_dtype)
+        total = None if brow is None else (brow.float() * w.Z).contiguous()
+        y = capi.gemm_bfp8b(x2, w.packed, w.N, bias=total, epilogue=epilogue, out_dtype=out_dtype)
         return y.view(*x.shape[:-3], 1, M, w.N)
     y = torch.empty((w.Z, M, w.N), dtype=out_dtype, device="cuda")
     for z in range(w.Z):
