@@ -37,6 +37,12 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+# where the `traffic` figures come from: counter summaries under profiles/, taken with the library built at this commit
+TRAFFIC_SOURCE = {"streaming": "profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt",
+                  "gemm": "profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt",
+                  "library_commit": "see the header of each file"}
+
+
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -45,7 +51,75 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     p.add_argument("--no-gemm", action="store_true", help="skip the GEMM / FFN section")
     p.add_argument("--eager-timing", action="store_true", help="time every launch eagerly, no HIP graph (for counter runs)")
+    p.add_argument("--gemm-only", action="store_true", help="skip the streaming section's secondary lines (fp32 sources, queue forms)")
+    p.add_argument("--power-probe", type=float, default=0.0, metavar="SECONDS",
+                   help="instead of the benchmark: run each 8192^3 GEMM form (fused, with workspace, the vendor library's plain bf16 "
+                        "GEMM through torch.matmul) back to back for SECONDS while rocm-smi is polled for clock and power; prints one JSON line")
     return p.parse_args()
+
+
+def power_probe(seconds, torch, capi):
+    """Sustained 8192^3 loops with clock and power samples: what the part settles at once it has warmed into its power limit."""
+    import re
+    import subprocess
+    import threading
+
+    F = capi.DataFormatCode
+    n = 8192
+    g = torch.Generator(device="cuda:0").manual_seed(30)
+    wp = capi.tilize_pack(torch.randn(1, 1, n, n, generator=g, device="cuda:0") * 0.02, F.Bfp8_b)
+    g = torch.Generator(device="cuda:0").manual_seed(31)
+    x = torch.randn(n, n, generator=g, device="cuda:0").bfloat16()
+    wb = (torch.randn(n, n, generator=g, device="cuda:0") * 0.02).bfloat16()
+    y = torch.empty(n, n, dtype=torch.bfloat16, device="cuda:0")
+    ws = torch.empty(capi.gemm_workspace_bytes(n, n, n), dtype=torch.uint8, device="cuda:0")
+    forms = {"fused Bfp8_b-weight GEMM": lambda: capi.gemm_bfp8b(x, wp, n, out=y),
+             "Bfp8_b-weight GEMM with a workspace (bf16 panel)": lambda: capi.gemm_bfp8b(x, wp, n, out=y, workspace=ws),
+             "vendor library, plain bf16 GEMM (torch.matmul)": lambda: torch.matmul(x, wb, out=y)}
+    out = {}
+    for name, fn in forms.items():
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        samples, stop = [], threading.Event()
+
+        def poll():
+            while not stop.is_set():
+                # socket power and the clock of each of the eight XCDs (their mean is what the matrix cores run at)
+                txt = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True).stdout
+                xcd = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK: (\d+) MHz", txt)]
+                watts = re.search(r"SOCKET_POWER: ([0-9.]+) W", txt)
+                samples.append((sum(xcd) / len(xcd) if xcd else None, float(watts.group(1)) if watts else None))
+                stop.wait(0.25)
+
+        th = threading.Thread(target=poll)
+        t0 = time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        launches = 0
+        th.start()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(50):
+                fn()
+            launches += 50
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        stop.set()
+        th.join()
+        ms = e0.elapsed_time(e1) / launches
+        late = samples[len(samples) // 2:]  # the second half of the run: the part has settled
+        clocks = sorted(c for c, _ in late if c)
+        watts = sorted(w for _, w in late if w)
+        tf = 2.0 * n ** 3 / ms / 1e9
+        out[name] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_of_2500": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "launches": launches,
+                     "xcd_clock_mhz_median": round(clocks[len(clocks) // 2]) if clocks else None,
+                     "socket_power_w_median": watts[len(watts) // 2] if watts else None,
+                     # what the matrix cores could do at the clock the part actually ran at: 256 CUs x 4 SIMDs x 1024 flop per clock
+                     "mfma_peak_at_that_clock_tflops": round(256 * 4 * 1024 * clocks[len(clocks) // 2] * 1e6 / 1e12, 1) if clocks else None}
+    cap = re.search(r"Max Graphics Package Power \(W\): ([0-9.]+)", subprocess.run(["rocm-smi", "--showmaxpower"], capture_output=True, text=True).stdout)
+    print(json.dumps({"power_probe_seconds": seconds, "shape": "8192 x 8192 x 8192", "max_package_power_w": float(cap.group(1)) if cap else None,
+                      "max_clock_mhz": 2400, "forms": out}))
 
 
 def time_kernel(fn, steps, warmup, torch):
@@ -120,6 +194,9 @@ def main():
     torch.cuda.set_device(0)
     capi.check(capi.lib().ttbfp_init(0))
     dev = "cuda:0"
+    if args.power_probe > 0:
+        power_probe(args.power_probe, torch, capi)
+        return
 
     # ---- streaming workload: bf16 [8,1,8192,8192], U(-8,8), seed 2 --------------------------------
     shape = (8, 1, 8192, 8192)
@@ -162,9 +239,25 @@ def main():
     }
     dominant = "tilize_pack_bf16_to_bfp8b" if pack_ms >= unpack_ms else "unpack_untilize_bfp8b_to_bf16"
 
+    # The headline certifies itself: outside the timed region, the bytes the timed launches left in `packed` and the
+    # floats in `back` are compared bit for bit with the CPU oracle on the first and the last 32-row band of the tensor.
+    import numpy as np
+
+    import oracle as O
+
+    band_bytes = (shape[3] // 32) * capi.tile_bytes(F.Bfp8_b)
+    for w_i, r0 in ((0, 0), (shape[0] - 1, shape[2] - 32)):
+        rows = x[w_i:w_i + 1, :, r0:r0 + 32].view(torch.int16).cpu().numpy().view(np.uint16)
+        want = O.tilize_pack(rows, O.Bfp8_b)
+        first = (w_i * (shape[2] // 32) + r0 // 32) * band_bytes
+        assert np.array_equal(packed[first:first + band_bytes].cpu().numpy(), want.reshape(-1)), "bench.py: packed bytes differ from the oracle"
+        want_back = O.unpack_untilize(want, O.Bfp8_b, (1, 1, 32, shape[3]), O.Float16_b)
+        got_back = back[w_i:w_i + 1, :, r0:r0 + 32].view(torch.int16).cpu().numpy().view(np.uint16)
+        assert np.array_equal(got_back, want_back), "bench.py: round-trip values differ from the oracle"
+
     # other source/destination pairs of the same kernels (secondary lines): fp32 [4,1,8192,8192], 1 GiB like the bf16 tensor
-    x32 = torch.randn(4, 1, 8192, 8192, device=dev)
-    for fmt, name in ((F.Bfp8_b, "bfp8b"), (F.Bfp4_b, "bfp4b"), (F.Bfp2_b, "bfp2b")):
+    x32 = torch.randn(4, 1, 8192, 8192, device=dev) if not args.gemm_only else None
+    for fmt, name in (((F.Bfp8_b, "bfp8b"), (F.Bfp4_b, "bfp4b"), (F.Bfp2_b, "bfp2b")) if not args.gemm_only else ()):
         pk = torch.empty(capi.packed_size(fmt, x32.shape), dtype=torch.uint8, device=dev)
         bk = torch.empty_like(x32)
         b = x32.numel() * 4 + pk.numel()
@@ -174,11 +267,11 @@ def main():
         ms, _ = time_kernel(lambda: capi.unpack_untilize(pk, fmt, x32.shape, out=bk), args.steps, args.warmup, torch)
         kernels[f"unpack_untilize_{name}_to_fp32"] = dict(ms=round(ms, 4), bytes=b,
                                                           roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
-    del x32, pk, bk
+    x32 = pk = bk = None
 
     # the same workload laid into the buffers of a queue: an 8 x 8 grid of 16 x 8 micro blocks of 2 x 4 tiles,
     # column-major micro-block order, without and with the 32-byte header + padding per tile
-    for header, name in ((0, "queue_g8x8_u2x4_c"), (1, "queue_g8x8_u2x4_c_headers")):
+    for header, name in (((0, "queue_g8x8_u2x4_c"), (1, "queue_g8x8_u2x4_c_headers")) if not args.gemm_only else ()):
         lay = capi.QueueLayout(8, 8, 16, 8, 2, 4, 1, header)
         qbytes = capi.queue_buffer_bytes(F.Bfp8_b, shape, lay) * 64
         qmem = torch.empty(qbytes, dtype=torch.uint8, device=dev)
@@ -221,7 +314,10 @@ def main():
                 out["eager_ms"] = round(eager_ms, 4)
             key = ("gemm_8192" if M == N == K == 8192 else "gemm_M%d" % M if N == K == 4096 else "") + ("_ws" if workspace else "")
             traffic = MEASURED_TRAFFIC_BYTES.get(key)
-            if M <= 32:  # weight streaming: HBM bound
+            # which roof bounds the shape: flops per minimum byte against the ridge of the two peaks (2500 TFLOP/s over 8 TB/s =
+            # 312 flop/B).  At N = K = 4096: M = 32 57, 64 113, 128 216 flop/B (HBM bound, the weight streams once), 512 656.
+            out["flop_per_byte"] = round(flops / min_bytes, 1)
+            if flops / min_bytes < MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
                 out["roofline"] = roofline("hbm", min_bytes / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", traffic)
             else:
                 out["roofline"] = roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", traffic)
@@ -272,10 +368,6 @@ def main():
     # ---- CPU baseline: the oracle on a bounded sample of the same workload ---------------------------
     cpu_baseline = None
     if not args.no_cpu_baseline:
-        import numpy as np
-
-        import oracle as O
-
         cores = max(1, min(16, os.cpu_count() or 1))
         sample_shape = (1, 1, 8192, 8192)  # one eighth of the workload
         xs = x[0:1].cpu().view(torch.int16).numpy().view(np.uint16)
@@ -307,18 +399,30 @@ def main():
             "single_thread_sample": "bf16 [1,1,1024,8192] slice x %d passes in %.1f s, 1 thread" % (reps1, dt1),
         }
         if not args.no_gemm:
-            # dequantize-then-fp32-matmul on the host cores (the golden evaluation), M = 512
+            # dequantize-then-fp32-matmul on the host cores (the golden evaluation) on config 4's seeded weight and activations,
+            # M = 512: the dequantization timed once, the matmul warmed and then timed apart from it
             torch.set_num_threads(cores)
-            wq = O.tilize_pack((np.random.default_rng(3).standard_normal((1, 1, 4096, 4096)) * 0.02).astype(np.float32),
-                               O.Bfp8_b, nthreads=cores)
-            a = torch.randn(512, 4096).bfloat16()
+            w4 = torch.randn(4096, 4096, generator=torch.Generator().manual_seed(3)) * 0.02
+            wq = O.tilize_pack(w4.view(1, 1, 4096, 4096).numpy(), O.Bfp8_b, nthreads=cores)
+            a = torch.randn(512, 4096, generator=torch.Generator().manual_seed(4)).bfloat16().float()
             t2 = time.perf_counter()
             wd = torch.from_numpy(O.dequant_weight(wq, 4096, 4096))
-            _ = a.float() @ wd
-            dt2 = time.perf_counter() - t2
-            cpu_baseline["gemm"] = {"value": round(2.0 * 512 * 4096 * 4096 / dt2 / 1e12, 4), "unit": "TFLOP/s",
+            dt_dequant = time.perf_counter() - t2
+            for _ in range(2):
+                _ = a @ wd
+            reps2, t3 = 0, time.perf_counter()
+            while True:
+                _ = a @ wd
+                reps2 += 1
+                dt2 = time.perf_counter() - t3
+                if dt2 >= 3.0:
+                    break
+            cpu_baseline["gemm"] = {"value": round(2.0 * 512 * 4096 * 4096 * reps2 / dt2 / 1e12, 4), "unit": "TFLOP/s",
                                     "cores": cores, "kind": "port",
-                                    "sample": "M=512, K=N=4096: oracle dequantize + torch fp32 matmul"}
+                                    "sample": "M=512, K=N=4096, config 4's weight (seed 3) and activations (seed 4): torch fp32 matmul on "
+                                              "the oracle-dequantized weight, %d warmed passes in %.1f s" % (reps2, dt2),
+                                    "dequantize_ms": round(dt_dequant * 1e3, 2),
+                                    "value_with_dequantize_each_call": round(2.0 * 512 * 4096 * 4096 / (dt2 / reps2 + dt_dequant) / 1e12, 4)}
 
     line = {
         "metric": "Bfp8_b pack/unpack GB/s (% HBM peak); Bfp8_b-weight GEMM TFLOP/s (% MFMA peak)",
@@ -331,12 +435,13 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u8",
+        "dtype": "bf16 <-> Bfp8_b (integer arithmetic on the 16-bit patterns; GEMM lines: bf16 x bf16 MFMA, fp32 accumulate)",
         "data": "synthetic",
         "config": {"workload": "streaming: bf16 [8,1,8192,8192] U(-8,8) seed 2 -> tilize+pack Bfp8_b -> "
                                "unpack+untilize bf16; one step = both kernels",
                    "algorithmic_bytes_per_step": bytes_pack + bytes_unpack},
         "roofline": dict(kernels[dominant]["roofline"], kernel=dominant),
+        "traffic_source": TRAFFIC_SOURCE,
         "cpu_baseline": cpu_baseline,
         "kernels": kernels,
         "gemm": gemm,

@@ -159,24 +159,23 @@ __device__ __forceinline__ void accumulator_settle()
 }
 
 // 16 bytes per lane from global memory (uniform base + per-lane 32-bit offset + OFFSET) straight into
-// LDS at M0 + OFFSET + lane * 16: the instruction offset applies to both addresses.  Four loads whose
-// LDS destinations are 1 KiB apart can therefore share one value of M0 (SET_M0 only on the first),
-// with the lane offsets prepared so that the global addresses come out right.
+// LDS at M0 + OFFSET + lane * 16: the instruction offset applies to both addresses.  The four loads of a
+// group, whose LDS destinations are 1 KiB apart, use one value of M0 and offsets 0, 1024, 2048, 3072, with the
+// lane offsets prepared so that the global addresses come out right.  Every load writes M0 itself, in the same
+// statement that uses it, and says so to the compiler (clobber): nothing the compiler may place between two
+// statements - it is free to use M0 for its own purposes - can then send a transfer to the wrong LDS address.
 // Issued as inline assembly on purpose: for the builtin the compiler cannot tell that the transfer
 // and the surrounding LDS accesses never overlap and drains all outstanding loads (vmcnt(0)) before
 // every following LDS instruction, which serializes the whole slab.  Completion is awaited
 // explicitly with wait_direct_loads() before the barrier that publishes the stage.
-template <int OFFSET, bool SET_M0>
+template <int OFFSET>
 __device__ __forceinline__ void direct_load_16(uint64_t base, uint32_t lane_offset, uint32_t lds_base)
 {
     static_assert(OFFSET >= 0 && OFFSET < 4096, "13-bit signed instruction offset");
-    if constexpr (SET_M0)
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%c3"
-                     :
-                     : "v"(lane_offset), "s"(base), "s"(lds_base), "n"(OFFSET)
-                     : "memory");
-    else
-        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%c2" : : "v"(lane_offset), "s"(base), "n"(OFFSET) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%c3"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_base), "n"(OFFSET)
+                 : "memory", "m0");
 }
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 // all but the LAST most recently issued loads (loads complete in order)
@@ -261,11 +260,9 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         const uint32_t chunk = (lane & 7) ^ (lane >> 3) ^ ((wave * XI + i) & 7u);
         x_off[i] = (i * 8 + (lane >> 3)) * K * 2 + chunk * 16 - (i % 4) * 1024;
     }
-    // Between two loads of a group of four nothing else may write M0; the compiler has no reason to
-    // (LDS instructions do not need it on this target) and the loads of a group sit in adjacent slots.
     auto load_x = [&](uint32_t slab, uint32_t stage, auto ic) {
         constexpr int I = decltype(ic)::value;
-        direct_load_16<(I % 4) * 1024, I % 4 == 0>(x_wave + (uint64_t)slab * (BK * 2), x_off[I],
+        direct_load_16<(I % 4) * 1024>(x_wave + (uint64_t)slab * (BK * 2), x_off[I],
                                                    lds_base + stage * STAGE + (wave * XI + I / 4 * 4) * 8 * A_ROW);
     };
 
@@ -275,7 +272,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     const uint32_t b_lane = lane * 16;
     auto load_b = [&](uint32_t slab, uint32_t stage, auto ic) {
         constexpr int I = decltype(ic)::value;
-        direct_load_16<(I % 4) * 1024, I % 4 == 0>(b_wave + (uint64_t)slab * S::B_BYTES + (I / 4) * 4096, b_lane,
+        direct_load_16<(I % 4) * 1024>(b_wave + (uint64_t)slab * S::B_BYTES + (I / 4) * 4096, b_lane,
                                                    lds_base + stage * STAGE + A_BYTES + wave * (S::B_BYTES / S::NW) + (I / 4) * 4096);
     };
 
