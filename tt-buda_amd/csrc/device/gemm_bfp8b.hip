@@ -2,10 +2,15 @@
 // weight streaming kernel, macro-tile aligned shapes -> the MFMA kernel of gemm_bfp8b_kernel.hpp in
 // one of two tile shapes, a row count that is not a multiple of 128 -> both (rows split), everything
 // else (N or K that do not suit the tiles) -> the bounds-checked general kernel.
+#include <cstdlib>
+
 #include "gemm_bfp8b_kernel.hpp"
 
 namespace ttbfp {
 
+#ifndef TTBFP_SLIM_BELOW_TILES
+#define TTBFP_SLIM_BELOW_TILES 256  // fewer 128 x 128 tiles than this: 128 x 64 tiles, twice as many workgroups
+#endif
 #ifndef TTBFP_BIG_MIN_TILES
 #define TTBFP_BIG_MIN_TILES 192  // fewer macro tiles than this leave too many of the 256 CUs idle
 #endif
@@ -15,6 +20,12 @@ hipError_t launch_gemm_bfp8b_general(uint32_t M, uint32_t N, uint32_t K, const v
 hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
                                     int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
 
+static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x 128), 3 (256 x 256 where it fits), 0 / unset: automatic
+{
+    static const int force = [] { const char *v = getenv("TTBFP_GEMM_TILE"); return v ? atoi(v) : 0; }();
+    return force;
+}
+
 static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
                                int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
 {
@@ -22,9 +33,14 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
     const bool f32 = y_fmt == kFloat32;
     // Large problems: 256 x 256 macro tiles (eight wavefronts); smaller ones 128 x 128 so that every CU gets work.
     const uint64_t big_tiles = (uint64_t)(M / 256) * (N / 256);
-    if (gemm_fits<BigShape>(M, N, K) && big_tiles >= TTBFP_BIG_MIN_TILES)
+    if (gemm_fits<BigShape>(M, N, K) && big_tiles >= TTBFP_BIG_MIN_TILES && force_tile() != 1 && force_tile() != 2)
         return f32 ? launch_gemm_bfp8b_big_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_big_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    const int force = force_tile();
+    const uint64_t small_tiles = (uint64_t)(M / 128) * (N / 128);
+    if (gemm_fits<SlimShape>(M, N, K) && (force == 1 || (force == 0 && small_tiles < TTBFP_SLIM_BELOW_TILES)))
+        return f32 ? launch_gemm_bfp8b_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
     if (gemm_fits<SmallShape>(M, N, K))
         return f32 ? launch_gemm_bfp8b_small_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_small_bf16(M, N, K, x, w, bias, epilogue, y, stream);

@@ -49,11 +49,12 @@ constexpr uint32_t kW8Tile = tile_bytes(kBfp8_b);
 
 __device__ __forceinline__ uint32_t swizzle_n(uint32_t n) { return n ^ (((n >> 3) ^ (n >> 6)) & 7u); }
 
-// One thread's share of a W slab: PW consecutive n x 8 consecutive k of one face.
-template <int PW>
+// One thread's share of a W slab: PW consecutive n x KH consecutive k of one face (KH = 8: a whole k chunk of the B
+// stage; KH = 4: its lower or upper half, for tiles so narrow that a whole chunk per thread would leave threads idle).
+template <int PW, int KH>
 struct WPatch {
-    uint32_t d[8][PW / 4];  // d[j][c]: datums of k = j, columns 4c .. 4c+3
-    uint2 e;                // shared exponents of k = 0..3 (.x) and 4..7 (.y)
+    uint32_t d[KH][PW / 4];  // d[j][c]: datums of k = j, columns 4c .. 4c+3
+    uint2 e;                 // shared exponents of k = 0..3 (.x) and, with KH = 8, 4..7 (.y)
 };
 
 // Hides a value from the optimizer (no instruction is emitted).  Without it the 0x7f mask is folded
@@ -89,14 +90,16 @@ struct Shape {
     static constexpr int NW = WM * WN, NT = 64 * NW;            // wavefronts, threads
     static constexpr int MB = BM / WM / 32, NB = BN / WN / 32;  // 32x32 blocks per wave in m and n
     static constexpr int XI = BM / 8 / NW;                      // direct X loads (8 rows each) per wave per slab
-    static constexpr int PW = 8 * BN / NT;                      // W columns per thread per slab (x 8 k)
+    static constexpr int PW = 8 * BN / NT >= 4 ? 8 * BN / NT : 4;  // W columns per thread per slab
+    static constexpr int KH = BK * BN / NT / PW;                   // ... x KH k: 8, or 4 for narrow tiles
     static constexpr uint32_t A_BYTES = BM * A_ROW, B_BYTES = (BK / 8) * BN * 16;
     static constexpr uint32_t STAGE = A_BYTES + B_BYTES;
     static_assert(NW == 4 || NW == 8, "one or two wavefronts per SIMD");
     static_assert(MB * NB <= 16 && (NW == 4 || MB * NB <= 8), "the accumulators of a SIMD's wavefronts must fit its AGPRs");
     static_assert(PW == 4 || PW == 8, "a thread dequantizes 4 or 8 columns");
+    static_assert(KH == 8 || (KH == 4 && PW == 4), "a thread dequantizes a whole k chunk, or half of one at four columns");
     static_assert(MB % 2 == 0, "operand addressing assumes an even number of m blocks per wave");
-    static_assert(MB + NB <= MB * NB, "one operand read per MFMA slot");
+    static_assert(MB + NB <= 2 * MB * NB, "at most two operand reads per MFMA slot");
 };
 
 // ---- accumulators ------------------------------------------------------------------------------------
@@ -168,6 +171,10 @@ __device__ __forceinline__ void accumulator_settle()
 // and the surrounding LDS accesses never overlap and drains all outstanding loads (vmcnt(0)) before
 // every following LDS instruction, which serializes the whole slab.  Completion is awaited
 // explicitly with wait_direct_loads() before the barrier that publishes the stage.
+// (M0 is a register the compiler reserves for itself: it warns that it will not save and restore it around the
+// statement, which is not wanted here either - the clobber is there to tell it that its own copy of M0, if any, is gone.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 template <int OFFSET>
 __device__ __forceinline__ void direct_load_16(uint64_t base, uint32_t lane_offset, uint32_t lds_base)
 {
@@ -177,6 +184,7 @@ __device__ __forceinline__ void direct_load_16(uint64_t base, uint32_t lane_offs
                  : "v"(lane_offset), "s"(base), "s"(lds_base), "n"(OFFSET)
                  : "memory", "m0");
 }
+#pragma clang diagnostic pop
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 // all but the LAST most recently issued loads (loads complete in order)
 template <int LAST>
@@ -218,7 +226,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
                                                            const uint8_t *__restrict__ Wp,
                                                            const uint16_t *__restrict__ bias, OutT *__restrict__ Y)
 {
-    constexpr int BM = S::BM, BN = S::BN, MB = S::MB, NB = S::NB, XI = S::XI, PW = S::PW;
+    constexpr int BM = S::BM, BN = S::BN, MB = S::MB, NB = S::NB, XI = S::XI, PW = S::PW, KH = S::KH;
     constexpr uint32_t A_BYTES = S::A_BYTES, STAGE = S::STAGE;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -277,21 +285,25 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     };
 
     // ---- W: this thread's patch inside a slab: columns w_n .. w_n+PW-1, k chunk w_kc (8 k each)
-    const uint32_t w_n = (tid % (BN / PW)) * PW, w_kc = tid / (BN / PW);
+    // (with KH = 4 two threads share a chunk: w_half says which four of its eight k this one holds)
+    const uint32_t w_n = (tid % (BN / PW)) * PW, w_kc = tid / (BN / PW) / (8 / KH), w_half = KH == 8 ? 0 : (tid / (BN / PW)) & 1;
     const uint32_t w_face = ((w_kc >> 1) & 1) * 2 + ((w_n >> 4) & 1), w_kh = w_kc & 1;
-    const uint32_t w_in_tile = w_face * 256 + w_kh * 128 + (w_n & 15);
+    const uint32_t w_in_tile = w_face * 256 + w_kh * 128 + w_half * 64 + (w_n & 15);
     const uint32_t w_key = ((w_n >> 3) ^ (w_n >> 6)) & 7u;
-    const uint32_t w_lds = A_BYTES + (w_kc * BN + (w_n & ~7u)) * 16;  // the 8-column group the patch lies in
+    const uint32_t w_lds = A_BYTES + (w_kc * BN + (w_n & ~7u)) * 16 + w_half * 8;  // the 8-column group the patch lies in
     const uint64_t w_slab_bytes = (uint64_t)(BK / kTile) * tiles_n * kW8Tile;
     const uint8_t *w_src = Wp + ((uint64_t)(w_kc >> 2) * tiles_n + n0 / kTile + w_n / kTile) * kW8Tile + (uint64_t)split * nslabs * w_slab_bytes;
 
     // Two register sets, set q holding slabs of parity q: while one is dequantized into LDS the loads
     // of the following slab are in flight into the other, a whole iteration ahead of their use.
-    WPatch<PW> wp[2];
-    auto fetch_w = [&](uint32_t slab, auto pc, auto uc) {  // unit 0: exponents, units 1..8: datum rows
+    WPatch<PW, KH> wp[2];
+    constexpr int WU = 1 + KH;  // fetch units per slab
+    auto fetch_w = [&](uint32_t slab, auto pc, auto uc) {  // unit 0: exponents, units 1..KH: datum rows
         constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
         const uint8_t *t = w_src + slab * w_slab_bytes;
-        if constexpr (U == 0) {
+        if constexpr (U == 0 && KH == 4) {
+            wp[P].e.x = *(const uint32_t *)(t + w_face * 16 + w_kh * 8 + w_half * 4);
+        } else if constexpr (U == 0) {
             wp[P].e = *(const uint2 *)(t + w_face * 16 + w_kh * 8);
         } else if constexpr (PW == 8) {
             const uint2 v = *(const uint2 *)(t + kExpSection + w_in_tile + (U - 1) * 16);
@@ -303,13 +315,13 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     };
 
     // ---- staging of a W register set into an LDS stage, cut into small units ----------------------
-    int w_exp[8];               // E - 133 of the patch's 8 rows
-    uint32_t w_mag[8][PW / 4];  // datum words with the sign bits cleared
+    int w_exp[KH];               // E - 133 of the patch's rows
+    uint32_t w_mag[KH][PW / 4];  // datum words with the sign bits cleared
     uint32_t w_col[4];          // the column being assembled: four bf16 pairs
     auto stage_exponents = [&](auto pc) {
         constexpr int P = decltype(pc)::value;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) w_exp[j] = (int)(((j < 4 ? wp[P].e.x : wp[P].e.y) >> (8 * (j & 3))) & 0xffu) - 133;
+        for (int j = 0; j < KH; ++j) w_exp[j] = (int)(((j < 4 ? wp[P].e.x : wp[P].e.y) >> (8 * (j & 3))) & 0xffu) - 133;
     };
     // The dequantization of a patch is cut into micro-steps of three to four instructions, one per
     // MFMA slot, whose operands were produced at least one slot earlier: a lone wavefront has nobody
@@ -319,12 +331,13 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     //   1: gather the sign bytes of both pairs, scale the first pair;
     //   2: scale the second pair, pack the first;
     //   3: pack the second pair, merge the signs, and with H == 1 store the column's eight k.
-    constexpr int NU = 4 * 2 * PW;  // micro-steps per slab
+    // With KH = 4 a thread holds one half of every column: G = I, and the four k are stored as one 64-bit vector.
+    constexpr int NU = 4 * (KH / 4) * PW;  // micro-steps per slab
     float q_f[4];
     uint32_t q_sgn[2], q_mag;
     auto dequant_step = [&](uint8_t *st, auto pc, auto uc) {
         constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
-        constexpr int G = U / 4, MS = U % 4, I = G / 2, H = G % 2, C = I / 4, B = I % 4, R = 4 * H;
+        constexpr int G = U / 4, MS = U % 4, I = G / (KH / 4), H = G % (KH / 4), C = I / 4, B = I % 4, R = 4 * H;
         constexpr uint32_t SIGN_SEL = 0x000c000cu | ((uint32_t)(4 + B) << 24) | ((uint32_t)B << 8);
         if constexpr (MS == 0) {
             if constexpr (B == 0) {
@@ -346,7 +359,9 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
             const uint32_t mag1 = __builtin_amdgcn_perm(__float_as_uint(q_f[3]), __float_as_uint(q_f[2]), 0x07060302u);
             w_col[2 * H] = (q_sgn[0] & 0x80008000u) | q_mag;
             w_col[2 * H + 1] = (q_sgn[1] & 0x80008000u) | mag1;
-            if constexpr (H == 1)  // the column is complete: store its eight k as one 128-bit vector
+            if constexpr (KH == 4)  // this thread's four k of the column
+                *(uint2 *)(st + w_lds + ((((w_n & 7u) + I) ^ w_key) * 16)) = make_uint2(w_col[0], w_col[1]);
+            else if constexpr (H == 1)  // the column is complete: store its eight k as one 128-bit vector
                 *(uint4 *)(st + w_lds + ((((w_n & 7u) + I) ^ w_key) * 16)) = make_uint4(w_col[0], w_col[1], w_col[2], w_col[3]);
         }
     };
@@ -367,12 +382,18 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
 
     bf16x8 fa[2][MB], fb[2][NB];
     // operand read U (0 .. MB+NB-1) of k step KS into fragment buffer BUF
-    auto read_frag = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) {
+    auto read_one = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) {
         constexpr int U = decltype(uc)::value, KS = decltype(ksc)::value, BUF = decltype(bufc)::value;
         if constexpr (U < MB)
             fa[BUF][U] = *(const bf16x8 *)(st + a_off[(KS + 2 * (U & 1)) & 3] + U * 32 * A_ROW);
-        else
+        else if constexpr (U < MB + NB)
             fb[BUF][U - MB] = *(const bf16x8 *)(st + b_off[U - MB] + KS * 2 * BN * 16);
+    };
+    // the operand reads of MFMA slot U: read U, and where a k step has fewer MFMAs than operands also read U + MB NB
+    auto read_frag = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) {
+        constexpr int U = decltype(uc)::value;
+        read_one(st, uc, ksc, bufc);
+        if constexpr (U < MB * NB) read_one(st, std::integral_constant<int, U + MB * NB>{}, ksc, bufc);
     };
 
     constexpr bool ALL_AGPRS = MB * NB > 8;
@@ -401,6 +422,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     constexpr int X_FIRST = SLOTS >= 32 && TOUCHED < 9 ? 9 : TOUCHED;
     constexpr int X_STEP = (SLOTS / 2 - X_FIRST) / XI > 1 ? (SLOTS / 2 - X_FIRST) / XI : 1;
     static_assert(X_FIRST + (XI - 1) * X_STEP < SLOTS, "every X load needs a slot");
+    static_assert(WU <= SLOTS, "every W fetch needs a slot");
 
     // One iteration (P = s & 1): k step 3 of slab s, then k steps 0..2 of slab s+1 (stage P^1).
     // With STAGING, slab s+2 is assembled in stage P meanwhile and a barrier publishes it at the end.
@@ -417,7 +439,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
                 constexpr int U = decltype(uc)::value, T = G * MF + U;
                 if constexpr (U < MB + NB) read_frag(cur, uc, integral_constant<int, G>{}, integral_constant<int, G & 1>{});
                 if constexpr (STAGING) {
-                    if constexpr (T < 9) fetch_w(w_slab, integral_constant<int, P ^ 1>{}, integral_constant<int, T>{});
+                    if constexpr (T < WU) fetch_w(w_slab, integral_constant<int, P ^ 1>{}, integral_constant<int, T>{});
                     if constexpr (T == 0) stage_exponents(pc);
                     static_for<NU>([&](auto kc) {  // micro-steps spread evenly over slots 1 .. SLOTS - 1
                         if constexpr (1 + decltype(kc)::value * (SLOTS - 1) / NU == T) dequant_step(dst, pc, kc);
@@ -479,19 +501,19 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         wait_direct_loads_except<(NSTAGE - 2) * (XI + BI)>();  // slabs 0 and 1 are needed first
     } else {
     static_for<XI>([&](auto ic) { load_x(0, 0, ic); });
-    static_for<9>([&](auto uc) { fetch_w(0, P0, uc); });
-    static_for<9>([&](auto uc) { fetch_w(last < 1 ? last : 1, P1, uc); });
+    static_for<WU>([&](auto uc) { fetch_w(0, P0, uc); });
+    static_for<WU>([&](auto uc) { fetch_w(last < 1 ? last : 1, P1, uc); });
     stage_exponents(P0);
     static_for<NU>([&](auto kc) { dequant_step(lds, P0, kc); });
     static_for<XI>([&](auto ic) { load_x(last < 1 ? last : 1, 1, ic); });
     stage_exponents(P1);
     static_for<NU>([&](auto kc) { dequant_step(lds + STAGE, P1, kc); });
-    static_for<9>([&](auto uc) { fetch_w(last < 2 ? last : 2, P0, uc); });
+    static_for<WU>([&](auto uc) { fetch_w(last < 2 ? last : 2, P0, uc); });
     }
     wait_direct_loads();
     __syncthreads();
     // k steps 0..2 of slab 0; the barrier after them frees stage 0 for slab 2
-    static_for<MB + NB>([&](auto uc) { read_frag(lds, uc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
+    static_for<MB + NB>([&](auto uc) { read_one(lds, uc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
     static_for<3>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
         k_step(integral_constant<int, G & 1>{}, [&](auto uc) {
@@ -600,6 +622,9 @@ hipError_t launch_shape(uint32_t M, uint32_t N, uint32_t K, const void *x, const
 #endif
 using BigShape = TTBFP_BIG_SHAPE;
 using SmallShape = Shape<128, 128, 2, 2>;
+// Half as wide: twice the workgroups for shapes whose 128 x 128 tiles leave CUs idle, and half the weights to dequantize
+// per workgroup and slab (a thread holds four k of four columns); three of them fit a CU.
+using SlimShape = Shape<128, 64, 2, 2>;
 
 // true if the problem can be cut into macro tiles of shape S
 template <typename S>
@@ -616,6 +641,8 @@ TTBFP_DECLARE_GEMM(big_f32);
 TTBFP_DECLARE_GEMM(big_bf16);
 TTBFP_DECLARE_GEMM(small_f32);
 TTBFP_DECLARE_GEMM(small_bf16);
+TTBFP_DECLARE_GEMM(slim_f32);
+TTBFP_DECLARE_GEMM(slim_bf16);
 TTBFP_DECLARE_GEMM(panel_f32);   // BigShape on a bf16 panel of W instead of the packed tiles
 TTBFP_DECLARE_GEMM(panel_bf16);
 TTBFP_DECLARE_GEMM(panel_small_f32);  // SmallShape on a panel made for 128-wide tiles

@@ -1,0 +1,6 @@
+// Bfp8_b-weight GEMM, macro tile SlimShape (128 x 64), Float16_b output: see gemm_bfp8b_kernel.hpp.
+#include "gemm_bfp8b_kernel.hpp"
+
+namespace ttbfp {
+TTBFP_DEFINE_GEMM(slim_bf16, SlimShape, uint16_t)
+}  // namespace ttbfp

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void unpack_untilize_blocks(const uint8_t *__r
     const uint8_t *tile_in = src + (QUEUE ? tile_offset(q, w, z, tr, tc) : tile * TB);
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-        if (c + j >= g.Cl) break;
+        if (c + j >= g.Cl) continue;  // narrowed away
         uint32_t bits;
         if constexpr (M != 0) {
             constexpr int ROW_BYTES = 16 * (M + 1) / 8;
