@@ -238,6 +238,13 @@ def main():
                                                                 MEASURED_TRAFFIC_BYTES["unpack_untilize"])),
     }
     dominant = "tilize_pack_bf16_to_bfp8b" if pack_ms >= unpack_ms else "unpack_untilize_bfp8b_to_bf16"
+    # yardstick, and the reference the traffic counters are scaled by: a plain device-to-device copy of the same 1 GiB tensor
+    spare = torch.empty_like(x)
+    copy_ms, _ = time_kernel(lambda: capi.check(capi.lib().ttbfp_memcpy_d2d(spare.data_ptr(), x.data_ptr(), elems * 2, capi._stream())),
+                             args.steps, args.warmup, torch)
+    del spare
+    kernels["reference_copy_1GiB_device_to_device"] = dict(ms=round(copy_ms, 4), bytes=elems * 4,
+                                                           roofline=roofline("hbm", elems * 4 / copy_ms / 1e6, HBM_PEAK_GBS, "GB/s"))
 
     # The headline certifies itself: outside the timed region, the bytes the timed launches left in `packed` and the
     # floats in `back` are compared bit for bit with the CPU oracle on the first and the last 32-row band of the tensor.
@@ -325,6 +332,16 @@ def main():
 
         gemm["north_star_8192"] = gemm_case(8192, 8192, 8192, 30)
         gemm["north_star_8192_with_workspace"] = gemm_case(8192, 8192, 8192, 30, workspace=True)
+        # reference point, not this library: the vendor library's plain bf16 GEMM on the same shape (no dequantization at all)
+        gg = torch.Generator(device=dev).manual_seed(31)
+        va = torch.randn(8192, 8192, generator=gg, device=dev).bfloat16()
+        vb = (torch.randn(8192, 8192, generator=gg, device=dev) * 0.02).bfloat16()
+        vy = torch.empty(8192, 8192, dtype=torch.bfloat16, device=dev)
+        vms, vmn = time_kernel(lambda: torch.matmul(va, vb, out=vy), args.steps, args.warmup, torch)
+        vtf = 2.0 * 8192 ** 3 / vms / 1e9
+        gemm["reference_vendor_plain_bf16_gemm_8192"] = dict(M=8192, N=8192, K=8192, ms=round(vms, 4), min_ms=round(vmn, 4), tflops=round(vtf, 2),
+                                                             roofline=roofline("mfma", vtf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        del va, vb, vy
         for M in (32, 512, 8192):
             gemm[f"config4_M{M}"] = gemm_case(M, 4096, 4096, 3)
         gemm["config4_M8192_with_workspace"] = gemm_case(8192, 4096, 4096, 3, workspace=True)

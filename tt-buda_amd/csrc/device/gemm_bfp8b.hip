@@ -11,6 +11,9 @@ namespace ttbfp {
 #ifndef TTBFP_SLIM_BELOW_TILES
 #define TTBFP_SLIM_BELOW_TILES 256  // fewer 128 x 128 tiles than this: 128 x 64 tiles, twice as many workgroups
 #endif
+#ifndef TTBFP_CUS
+#define TTBFP_CUS 256  // compute units of the part this library is built for (MI355X)
+#endif
 #ifndef TTBFP_BIG_MIN_TILES
 #define TTBFP_BIG_MIN_TILES 192  // fewer macro tiles than this leave too many of the 256 CUs idle
 #endif
@@ -38,9 +41,17 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
                    : launch_gemm_bfp8b_big_bf16(M, N, K, x, w, bias, epilogue, y, stream);
     const int force = force_tile();
     const uint64_t small_tiles = (uint64_t)(M / 128) * (N / 128);
-    if (gemm_fits<SlimShape>(M, N, K) && (force == 1 || (force == 0 && small_tiles < TTBFP_SLIM_BELOW_TILES)))
+    static const int ring = [] { const char *v = getenv("TTBFP_GEMM_RING"); return v ? atoi(v) : 1; }();  // tuning aid: 0 = two-stage form only
+    if (gemm_fits<SlimShape>(M, N, K) && (force == 1 || (force == 0 && small_tiles < TTBFP_SLIM_BELOW_TILES))) {
+        // At most one workgroup per CU: nothing else hides a workgroup's trips to memory, so the form with rings (loads
+        // issued two iterations ahead) wins - 512 x 4096 x 4096: 38 against 49 us.  With more workgroups than CUs the rings'
+        // LDS would cost the second and third workgroup of a CU, which hide latency better than the rings do.
+        if (ring && 2 * small_tiles <= TTBFP_CUS)
+            return f32 ? launch_gemm_bfp8b_ring_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
+                       : launch_gemm_bfp8b_ring_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
         return f32 ? launch_gemm_bfp8b_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    }
     if (gemm_fits<SmallShape>(M, N, K))
         return f32 ? launch_gemm_bfp8b_small_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_small_bf16(M, N, K, x, w, bias, epilogue, y, stream);

@@ -220,7 +220,15 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v)
 // SPLITK: the grid's y dimension cuts K into gridDim.y equal runs of slabs; workgroup (tile, j) multiplies run j only
 // and writes its fp32 partial tile into plane j of Y ([gridDim.y][M][N], no bias, no epilogue), for
 // gemm_bfp8b_splitk.hip to add up.  For shapes whose tiles do not fill the CUs.
-template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL = false, bool SPLITK = false>
+//
+// RING (= LA, the depth of the rings; 0: off): the form for tiles whose iteration is shorter than a trip to memory (the
+// 128-wide and 64-wide tiles on four wavefronts).  With two stages a slab's loads are issued and awaited inside one
+// iteration, so every slab costs that trip.  Here X goes into a ring of LA A stages and the packed bytes of W - two tile
+// rows of BN / 32 tiles, contiguous runs in HBM - by direct loads into a ring of LA raw areas, both LA - 2 iterations before
+// anything needs them; the dequantization reads its patch out of the raw area (LDS reads, which the compiler counts apart from
+// loads) into the B stage two iterations ahead as before.  All loads from memory are then direct loads in issue order,
+// and the one wait per iteration names exactly how many of the youngest may stay in flight.
+template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL = false, bool SPLITK = false, int RING = 0>
 __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t N, uint32_t K, int epilogue,
                                                            const uint16_t *__restrict__ X,
                                                            const uint8_t *__restrict__ Wp,
@@ -234,8 +242,11 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave / S::WN, wn = wave % S::WN;
     // Macro tile of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin and each XCD has
-    // its own L2, so when the tile grid allows it the 32 tiles an XCD works on at a time form a
-    // 4 (m) x 8 (n) block: its X rows and W columns are then fetched into that L2 once for 32 tiles.
+    // its own L2, so the tiles an XCD works on at a time should be neighbours: their X rows and W columns are then
+    // fetched into that L2 once for all of them.  When the tile grid allows it (XCD_BLOCKS) the 32 tiles an XCD works on at
+    // a time form a 4 (m) x 8 (n) block.  Any other grid is walked in panels of eight tile columns, down the rows inside a
+    // panel, and every XCD takes one contiguous eighth of that walk (the launch rounds the grid up to a multiple of
+    // eight; the workgroups past the end leave at once, before any barrier).
     uint32_t tile_m, tile_n;
     {
         const uint32_t gm = M / BM, gn = N / BN;
@@ -244,14 +255,23 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
             const uint32_t block = (id / 256) * 8 + id % 8, j = (id / 8) % 32;  // block of this XCD, tile inside it
             tile_m = (block % (gm / 4)) * 4 + j / 8;
             tile_n = (block / (gm / 4)) * 8 + j % 8;
-        } else {
+        } else if (SPLITK) {
             tile_m = id / gn;
             tile_n = id % gn;
+        } else {
+            const uint32_t tiles = gm * gn, share = (tiles + 7) / 8;
+            const uint32_t v = (id % 8) * share + id / 8;  // place in the walk
+            if (v >= tiles) return;
+            const uint32_t panel = v / (gm * 8), r = v - panel * (gm * 8);
+            const uint32_t width = gn - panel * 8 < 8 ? gn - panel * 8 : 8;
+            tile_m = r / width;
+            tile_n = panel * 8 + r % width;
         }
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     const uint32_t tiles_n = N / kTile;
     static_assert(!(SPLITK && PANEL) && (!SPLITK || sizeof(OutT) == 4), "k split: packed W, fp32 partial sums");
+    static_assert(RING == 0 || (RING >= 3 && !PANEL && !SPLITK && S::NW == 4), "rings: three or more stages, packed W, four wavefronts");
     const uint32_t split = SPLITK ? blockIdx.y : 0;
     const uint32_t nslabs = SPLITK ? K / BK / gridDim.y : K / BK;  // slabs split * nslabs .. + nslabs - 1
     if constexpr (SPLITK) Y += (uint64_t)split * M * N;
@@ -366,6 +386,52 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         }
     };
 
+    // ---- rings (RING): LDS = [LA A stages][two B stages][LA raw areas]; slab t uses A stage and raw area t % LA ---------
+    constexpr int LA = RING > 0 ? RING : 2;
+    constexpr uint32_t A_RING = LA * A_BYTES;
+    constexpr uint32_t RUN_BYTES = (BN / kTile) * kW8Tile;           // the tiles of one tile row that the macro tile spans
+    constexpr uint32_t RAW_CHUNKS = 2 * RUN_BYTES / 16;              // 16-byte pieces of a slab's two runs
+    constexpr uint32_t CPW = RAW_CHUNKS / S::NW;                     // pieces per wavefront
+    constexpr int WI = (CPW + 63) / 64;                              // direct loads per wavefront and slab
+    // the last load of a wavefront reaches past its share: into the next wavefront's (the same bytes, fetched twice) and,
+    // for the last wavefront, past the end of the area, which therefore carries that much padding
+    constexpr uint32_t RAW_PITCH = 2 * RUN_BYTES + (WI * 64 - CPW) * 16;
+    static_assert(RAW_CHUNKS % S::NW == 0 && RAW_PITCH % 16 == 0, "raw area: whole pieces per wavefront");
+    constexpr uint32_t RAW_BASE = A_RING + 2 * S::B_BYTES;
+    uint32_t raw_off[WI];  // offset of this lane's piece from the first tile of the slab (pieces past the end: the last one again)
+#pragma unroll
+    for (int i = 0; i < WI; ++i) {
+        const uint32_t c = wave * CPW + i * 64 + lane, cc = c < RAW_CHUNKS ? c : RAW_CHUNKS - 1;
+        const uint32_t run = cc / (RUN_BYTES / 16), within = cc % (RUN_BYTES / 16);
+        raw_off[i] = run * tiles_n * kW8Tile + within * 16;
+    }
+    const uint64_t raw_wave = uniform64((uint64_t)(uintptr_t)Wp + (uint64_t)(n0 / kTile) * kW8Tile);
+    auto load_x_ring = [&](uint32_t slab, uint32_t slot, auto ic) {
+        constexpr int I = decltype(ic)::value;
+        direct_load_16<(I % 4) * 1024>(x_wave + (uint64_t)slab * (BK * 2), x_off[I], lds_base + slot * A_BYTES + (wave * XI + I / 4 * 4) * 8 * A_ROW);
+    };
+    auto load_raw = [&](uint32_t slab, uint32_t slot, auto ic) {
+        constexpr int I = decltype(ic)::value;
+        direct_load_16<0>(raw_wave + (uint64_t)slab * w_slab_bytes, raw_off[I], lds_base + RAW_BASE + slot * RAW_PITCH + (wave * CPW + I * 64) * 16);
+    };
+    // this thread's patch out of a raw area into register set 0: the same units as fetch_w
+    const uint32_t raw_patch = (w_kc >> 2) * RUN_BYTES + (w_n / kTile) * kW8Tile;
+    auto fetch_w_ring = [&](uint32_t slot, auto uc) {
+        constexpr int U = decltype(uc)::value;
+        const uint8_t *t = lds + RAW_BASE + slot * RAW_PITCH + raw_patch;
+        if constexpr (U == 0 && KH == 4) {
+            wp[0].e.x = *(const uint32_t *)(t + w_face * 16 + w_kh * 8 + w_half * 4);
+        } else if constexpr (U == 0) {
+            wp[0].e = *(const uint2 *)(t + w_face * 16 + w_kh * 8);
+        } else if constexpr (PW == 8) {
+            const uint2 v = *(const uint2 *)(t + kExpSection + w_in_tile + (U - 1) * 16);
+            wp[0].d[U - 1][0] = v.x;
+            wp[0].d[U - 1][PW / 4 - 1] = v.y;
+        } else {
+            wp[0].d[U - 1][0] = *(const uint32_t *)(t + kExpSection + w_in_tile + (U - 1) * 16);
+        }
+    };
+
     // ---- operand fragment addresses of this lane (within a stage) ---------------------------------
     // A: row m = wm (BM/WM) + 32 mb + (lane & 31), logical chunk 2 ks + (lane >> 5).  The stored chunk is
     // chunk ^ key(m); key(m) = ((lane & 7) ^ ((lane >> 3) & 3)) ^ 4 (mb & 1), so the four values of
@@ -382,19 +448,22 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
 
     bf16x8 fa[2][MB], fb[2][NB];
     // operand read U (0 .. MB+NB-1) of k step KS into fragment buffer BUF
-    auto read_one = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) {
+    // (sta: where the A stage begins; stb: A_BYTES before the B stage - in the two-stage forms both are the stage itself)
+    auto read_one2 = [&](const uint8_t *sta, const uint8_t *stb, auto uc, auto ksc, auto bufc) {
         constexpr int U = decltype(uc)::value, KS = decltype(ksc)::value, BUF = decltype(bufc)::value;
         if constexpr (U < MB)
-            fa[BUF][U] = *(const bf16x8 *)(st + a_off[(KS + 2 * (U & 1)) & 3] + U * 32 * A_ROW);
+            fa[BUF][U] = *(const bf16x8 *)(sta + a_off[(KS + 2 * (U & 1)) & 3] + U * 32 * A_ROW);
         else if constexpr (U < MB + NB)
-            fb[BUF][U - MB] = *(const bf16x8 *)(st + b_off[U - MB] + KS * 2 * BN * 16);
+            fb[BUF][U - MB] = *(const bf16x8 *)(stb + b_off[U - MB] + KS * 2 * BN * 16);
     };
+    auto read_one = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) { read_one2(st, st, uc, ksc, bufc); };
     // the operand reads of MFMA slot U: read U, and where a k step has fewer MFMAs than operands also read U + MB NB
-    auto read_frag = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) {
+    auto read_frag2 = [&](const uint8_t *sta, const uint8_t *stb, auto uc, auto ksc, auto bufc) {
         constexpr int U = decltype(uc)::value;
-        read_one(st, uc, ksc, bufc);
-        if constexpr (U < MB * NB) read_one(st, std::integral_constant<int, U + MB * NB>{}, ksc, bufc);
+        read_one2(sta, stb, uc, ksc, bufc);
+        if constexpr (U < MB * NB) read_one2(sta, stb, std::integral_constant<int, U + MB * NB>{}, ksc, bufc);
     };
+    auto read_frag = [&](const uint8_t *st, auto uc, auto ksc, auto bufc) { read_frag2(st, st, uc, ksc, bufc); };
 
     constexpr bool ALL_AGPRS = MB * NB > 8;
     static_for<MB * NB * 16>([&](auto rc) { accumulator_clear<decltype(rc)::value, ALL_AGPRS>(); });
@@ -485,12 +554,95 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         __syncthreads();
     };
 
+    // The ring form of an iteration (P = s & 1): the same four k steps, A operands out of slab s + 1's A stage, B out of
+    // B stage P ^ 1.  Meanwhile slab s + 2 is dequantized out of its raw area into B stage P (the patch is read in the first
+    // slot, the micro-steps follow from the third on), X of slab s + LA goes into the A stage slab s has just left and the
+    // raw bytes of slab s + LA + 1 into the area slab s + 1 left one iteration ago.  At the end X of slab s + 2 and the raw
+    // bytes of slab s + 3 must have landed: they were issued LA - 2 iterations ago, so the loads of the iterations since
+    // then - (LA - 2) (XI + WI) of them, the youngest - may stay in flight.
+    constexpr int RING_FIRST = 2;  // first slot with micro-steps: the patch reads of slot 0 have had a slot to land
+    auto slot_of = [&](uint32_t slab) { return slab % LA; };
+    auto iteration_ring = [&](uint32_t s, auto pc, auto stagec) {
+        constexpr int P = decltype(pc)::value;
+        constexpr bool STAGING = decltype(stagec)::value;  // false: no slab s + 2 to dequantize
+        const uint8_t *cur_a = lds + slot_of(s + 1) * A_BYTES;
+        const uint8_t *cur_b = lds + A_RING + (P ^ 1) * S::B_BYTES - A_BYTES;
+        uint8_t *dst_b = lds + A_RING + P * S::B_BYTES - A_BYTES;
+        const uint32_t x_slab = s + LA < nslabs ? s + LA : nslabs - 1, raw_slab = s + LA + 1 < nslabs ? s + LA + 1 : nslabs - 1;
+        const uint32_t a_dst = slot_of(s), raw_dst = slot_of(s + 1), raw_src = slot_of(s + 2);
+        static_for<4>([&](auto gc) {
+            constexpr int G = decltype(gc)::value;
+            k_step(integral_constant<int, (G + 1) & 1>{}, [&](auto uc) {
+                constexpr int U = decltype(uc)::value, T = G * MF + U;
+                if constexpr (U < MB + NB) read_frag2(cur_a, cur_b, uc, integral_constant<int, G>{}, integral_constant<int, G & 1>{});
+                if constexpr (STAGING) {
+                    if constexpr (T == 0) static_for<WU>([&](auto fc) { fetch_w_ring(raw_src, fc); });
+                    if constexpr (T == RING_FIRST - 1) stage_exponents(integral_constant<int, 0>{});
+                    static_for<NU>([&](auto kc) {
+                        if constexpr (RING_FIRST + decltype(kc)::value * (SLOTS - RING_FIRST) / NU == T) dequant_step(dst_b, integral_constant<int, 0>{}, kc);
+                    });
+                }
+                static_for<XI>([&](auto ic) {
+                    if constexpr (1 + decltype(ic)::value * ((SLOTS - 2) / (XI + WI)) == T) load_x_ring(x_slab, a_dst, ic);
+                });
+                static_for<WI>([&](auto ic) {
+                    if constexpr (1 + (XI + decltype(ic)::value) * ((SLOTS - 2) / (XI + WI)) == T) load_raw(raw_slab, raw_dst, ic);
+                });
+            });
+        });
+        wait_direct_loads_except<(LA - 2) * (XI + WI)>();
+        __syncthreads();
+    };
+
     // prologue: slabs 0 and 1 into the two stages, W of slab 2 into register set 0, first operands
     constexpr integral_constant<int, 0> P0{};
     constexpr integral_constant<int, 1> P1{};
     constexpr integral_constant<bool, true> STAGE_ON{};
     constexpr integral_constant<bool, false> STAGE_OFF{};
     const uint32_t last = nslabs - 1;
+    if constexpr (RING > 0) {
+        static_assert((SLOTS - 2) / (XI + WI) >= 1 && (LA - 2) * (XI + WI) < 64, "every direct load needs a slot; vmcnt is a 6-bit counter");
+        // X and the raw bytes of slabs 0 .. LA - 1 (past the end: the last slab again, unused)
+        static_for<LA>([&](auto sc) {
+            constexpr uint32_t SL = decltype(sc)::value;
+            static_for<XI>([&](auto ic) { load_x_ring(last < SL ? last : SL, SL, ic); });
+            static_for<WI>([&](auto ic) { load_raw(last < SL ? last : SL, SL, ic); });
+        });
+        wait_direct_loads();
+        __syncthreads();
+        // slabs 0 and 1 dequantized into the two B stages
+        static_for<2>([&](auto sc) {
+            constexpr uint32_t SL = decltype(sc)::value;
+            static_for<WU>([&](auto fc) { fetch_w_ring(SL % LA, fc); });
+            stage_exponents(P0);
+            static_for<NU>([&](auto kc) { dequant_step(lds + A_RING + SL * S::B_BYTES - A_BYTES, P0, kc); });
+        });
+        __syncthreads();
+        // raw area 0 is free again: slab LA (the main loop goes on with slab LA + 1 in its first iteration)
+        static_for<WI>([&](auto ic) { load_raw(last < LA ? last : LA, 0, ic); });
+        // k steps 0..2 of slab 0; the barrier after them frees B stage 0 for slab 2
+        const uint8_t *b0 = lds + A_RING - A_BYTES;
+        static_for<MB + NB>([&](auto uc) { read_one2(lds, b0, uc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
+        static_for<3>([&](auto gc) {
+            constexpr int G = decltype(gc)::value;
+            k_step(integral_constant<int, G & 1>{}, [&](auto uc) {
+                if constexpr (decltype(uc)::value < MB + NB) read_frag2(lds, b0, uc, integral_constant<int, G + 1>{}, integral_constant<int, (G + 1) & 1>{});
+            });
+        });
+        __syncthreads();
+        uint32_t s = 0;
+        for (; s + 3 < nslabs; s += 2) {
+            iteration_ring(s, P0, STAGE_ON);
+            iteration_ring(s + 1, P1, STAGE_ON);
+        }
+        if (nslabs - s == 3) {
+            iteration_ring(s, P0, STAGE_ON);
+            iteration_ring(s + 1, P1, STAGE_OFF);
+        } else if (nslabs - s == 2) {
+            iteration_ring(s, P0, STAGE_OFF);
+        }
+        wait_direct_loads();  // nothing may still be on its way into LDS when the workgroup ends
+    } else {
     if constexpr (PANEL) {
         static_assert(1 + XI + BI < SLOTS, "every direct load needs a slot");
         static_for<NSTAGE>([&](auto sc) {  // slabs 0 .. NSTAGE-1 (past the end: the last slab again, unused)
@@ -541,6 +693,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         iteration(s, P0, STAGE_OFF);
     }
     }
+    }
     k_step(P1, [&](auto) {});  // k step 3 of the last slab
 
     // D layout of the 32x32 MFMA: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
@@ -573,10 +726,46 @@ hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, const void *x, const 
     static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (attr != hipSuccess) return attr;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
-    if (tiles > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles), dim3(S::NT), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
+    if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
+    const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);  // the walk in eighths: see the kernel
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
     return hipGetLastError();
+}
+
+// LDS of the ring form: LA A stages, two B stages, LA raw areas (the arithmetic of the kernel's RAW_PITCH)
+template <typename S, int LA>
+constexpr uint32_t ring_lds_bytes()
+{
+    constexpr uint32_t run = (S::BN / kTile) * kW8Tile, cpw = 2 * run / 16 / S::NW, wi = (cpw + 63) / 64;
+    return LA * S::A_BYTES + 2 * S::B_BYTES + LA * (2 * run + (wi * 64 - cpw) * 16);
+}
+
+template <typename S, typename OutT, bool XCD_BLOCKS, int LA>
+hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
+                            void *y, hipStream_t stream)
+{
+    constexpr uint32_t smem = ring_lds_bytes<S, LA>();
+    static_assert(smem <= 160 * 1024, "LDS of a CU");
+    auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, false, false, LA>;
+    static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (attr != hipSuccess) return attr;
+    const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
+    if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
+    const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
+                       (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
+    return hipGetLastError();
+}
+
+template <typename S, typename OutT, int LA>
+hipError_t launch_shape_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
+                             void *y, hipStream_t stream)
+{
+    const uint32_t gm = M / S::BM, gn = N / S::BN;
+    if (gm % 4 == 0 && gn % 8 == 0 && ((gm / 4) * (gn / 8)) % 8 == 0)
+        return launch_tile_ring<S, OutT, true, LA>(M, N, K, x, w, bias, epilogue, y, stream);
+    return launch_tile_ring<S, OutT, false, LA>(M, N, K, x, w, bias, epilogue, y, stream);
 }
 
 // k split: `splits` workgroups per tile, fp32 partial planes [splits][M][N] at `partials`
@@ -643,12 +832,16 @@ TTBFP_DECLARE_GEMM(small_f32);
 TTBFP_DECLARE_GEMM(small_bf16);
 TTBFP_DECLARE_GEMM(slim_f32);
 TTBFP_DECLARE_GEMM(slim_bf16);
+TTBFP_DECLARE_GEMM(ring_slim_f32);  // SlimShape in the ring form
+TTBFP_DECLARE_GEMM(ring_slim_bf16);
 TTBFP_DECLARE_GEMM(panel_f32);   // BigShape on a bf16 panel of W instead of the packed tiles
 TTBFP_DECLARE_GEMM(panel_bf16);
 TTBFP_DECLARE_GEMM(panel_small_f32);  // SmallShape on a panel made for 128-wide tiles
 TTBFP_DECLARE_GEMM(panel_small_bf16);
 #define TTBFP_DEFINE_PANEL_GEMM(NAME, SHAPE, OUT_T)                                                                    \
     TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, true>(M, N, K, x, w, bias, epilogue, y, stream); }
+#define TTBFP_DEFINE_RING_GEMM(NAME, SHAPE, OUT_T, LA)                                                                 \
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA>(M, N, K, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_GEMM(NAME, SHAPE, OUT_T)                                                                          \
     TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T>(M, N, K, x, w, bias, epilogue, y, stream); }
 
