@@ -23,7 +23,7 @@ hipError_t launch_gemm_bfp8b_general(uint32_t M, uint32_t N, uint32_t K, const v
 hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
                                     int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
 
-static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x 128), 3 (256 x 256 where it fits), 0 / unset: automatic
+static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x 128), 3 (256 x 256 where it fits), all on two stages; 0 / unset: automatic
 {
     static const int force = [] { const char *v = getenv("TTBFP_GEMM_TILE"); return v ? atoi(v) : 0; }();
     return force;
@@ -39,19 +39,30 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
     if (gemm_fits<BigShape>(M, N, K) && big_tiles >= TTBFP_BIG_MIN_TILES && force_tile() != 1 && force_tile() != 2)
         return f32 ? launch_gemm_bfp8b_big_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_big_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    // Fewer tiles than that: which tile and form, by how many workgroups a CU gets.
+    //   at most one 128 x 64 workgroup per CU: that tile with two pipelines per workgroup on rings (K a multiple of 128;
+    //     else one pipeline on rings) - 512 x 4096 x 4096: 37 us, one pipeline on rings 41, on two stages 49, 128 x 128 54;
+    //   else at most one 128 x 128 workgroup per CU: that tile on two stages with two pipelines (K a multiple of 128) -
+    //     3072 x 1024 x 4096: 44.5 us against 53 for 384 workgroups of 128 x 64, 512 x 8192 x 2048: 29 against 33;
+    //   else 128 x 64 on two stages below 256 tiles of 128 x 128 (three workgroups fit a CU), 128 x 128 above.
+    // TTBFP_GEMM_TILE (1: 128 x 64 on two stages, 2: 128 x 128 on two stages, 3: 256 x 256 where it fits) and
+    // TTBFP_GEMM_PIPELINES=1 (no workgroup with two pipelines) are tuning aids for measurements and override this.
     const int force = force_tile();
-    const uint64_t small_tiles = (uint64_t)(M / 128) * (N / 128);
-    static const int ring = [] { const char *v = getenv("TTBFP_GEMM_RING"); return v ? atoi(v) : 1; }();  // tuning aid: 0 = two-stage form only
-    if (gemm_fits<SlimShape>(M, N, K) && (force == 1 || (force == 0 && small_tiles < TTBFP_SLIM_BELOW_TILES))) {
-        // At most one workgroup per CU: nothing else hides a workgroup's trips to memory, so the form with rings (loads
-        // issued two iterations ahead) wins - 512 x 4096 x 4096: 38 against 49 us.  With more workgroups than CUs the rings'
-        // LDS would cost the second and third workgroup of a CU, which hide latency better than the rings do.
-        if (ring && 2 * small_tiles <= TTBFP_CUS)
-            return f32 ? launch_gemm_bfp8b_ring_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                       : launch_gemm_bfp8b_ring_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    static const bool duo = [] { const char *v = getenv("TTBFP_GEMM_PIPELINES"); return !v || atoi(v) != 1; }();
+    const uint64_t small_tiles = (uint64_t)(M / 128) * (N / 128), slim_tiles = (uint64_t)(M / 128) * (N / 64);
+    if (force == 0 && gemm_fits<SlimShape>(M, N, K) && slim_tiles <= TTBFP_CUS) {
+        if (duo && K % 128 == 0)
+            return f32 ? launch_gemm_bfp8b_duo_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
+                       : launch_gemm_bfp8b_duo_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+        return f32 ? launch_gemm_bfp8b_ring_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_ring_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    }
+    if (force == 0 && duo && gemm_fits<SmallShape>(M, N, K) && small_tiles <= TTBFP_CUS && K % 128 == 0)
+        return f32 ? launch_gemm_bfp8b_duo_small_f32(M, N, K, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_duo_small_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    if (gemm_fits<SlimShape>(M, N, K) && (force == 1 || (force == 0 && small_tiles < TTBFP_SLIM_BELOW_TILES)))
         return f32 ? launch_gemm_bfp8b_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
-    }
     if (gemm_fits<SmallShape>(M, N, K))
         return f32 ? launch_gemm_bfp8b_small_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_small_bf16(M, N, K, x, w, bias, epilogue, y, stream);

@@ -17,7 +17,9 @@
 // and must be spread evenly: the loop is written as slots of {one MFMA + a small unit of side work}
 // with the scheduler fenced at every slot boundary.
 // One iteration runs from barrier to barrier and holds 4 k steps: the last k step of slab s (its
-// operands were read before the barrier) and k steps 0..2 of slab s+1.  Stage s&1 is dead from the
+// operands were read before the barrier) and k steps 0..2 of slab s+1 - or, where a k step has so few MFMAs that
+// its operands must be read two k steps ahead (Shape::AHEAD), the last two of slab s and the first two of slab s+1;
+// either way an iteration reads all four k steps of slab s+1 and nothing else.  Stage s&1 is dead from the
 // barrier on, so during the whole iteration
 //   * X of slab s+2 goes from global memory straight into it (global_load_lds_dwordx4, no registers);
 //   * W of slab s+2, fetched into registers one iteration earlier, is dequantized into it;
@@ -47,7 +49,16 @@ constexpr int BK = 64;
 constexpr int A_ROW = BK * 2;  // bytes per A row in LDS
 constexpr uint32_t kW8Tile = tile_bytes(kBfp8_b);
 
-__device__ __forceinline__ uint32_t swizzle_n(uint32_t n) { return n ^ (((n >> 3) ^ (n >> 6)) & 7u); }
+// Where column n of a B stage sits inside its group of eight columns: slot (n & 7) ^ key(n / 8).  A 128-bit operand read
+// takes 16 consecutive columns of one k chunk per pass and is free of bank conflicts under any key; the key is chosen for
+// the stores of the dequantization.  Whole chunks (128-bit stores, one pass = column I of 16 groups): the keys of the eight
+// even and of the eight odd groups must differ, which g ^ (g >> 3) gives.  Half chunks (HALF: 64-bit stores, one pass =
+// columns I and I + 4 of the 8 groups of a 64-column stage, both halves): the keys of the four even and of the four odd
+// groups must differ in their low two bits, which g ^ (g >> 2) gives.
+template <bool HALF = false>
+__device__ __forceinline__ uint32_t swizzle_key(uint32_t n) { return HALF ? ((n >> 3) ^ (n >> 5)) & 7u : ((n >> 3) ^ (n >> 6)) & 7u; }
+template <bool HALF = false>
+__device__ __forceinline__ uint32_t swizzle_n(uint32_t n) { return n ^ swizzle_key<HALF>(n); }
 
 // One thread's share of a W slab: PW consecutive n x KH consecutive k of one face (KH = 8: a whole k chunk of the B
 // stage; KH = 4: its lower or upper half, for tiles so narrow that a whole chunk per thread would leave threads idle).
@@ -97,9 +108,15 @@ struct Shape {
     static_assert(NW == 4 || NW == 8, "one or two wavefronts per SIMD");
     static_assert(MB * NB <= 16 && (NW == 4 || MB * NB <= 8), "the accumulators of a SIMD's wavefronts must fit its AGPRs");
     static_assert(PW == 4 || PW == 8, "a thread dequantizes 4 or 8 columns");
-    static_assert(KH == 8 || (KH == 4 && PW == 4), "a thread dequantizes a whole k chunk, or half of one at four columns");
+    static_assert(KH == 8 || (KH == 4 && PW == 4 && BN == 64), "a thread dequantizes a whole k chunk, or half of one at four columns of a 64-column stage");
     static_assert(MB % 2 == 0, "operand addressing assumes an even number of m blocks per wave");
     static_assert(MB + NB <= 2 * MB * NB, "at most two operand reads per MFMA slot");
+    // How many k steps ahead of its MFMAs a k step's operands are read from LDS.  One step is time enough where a k step has
+    // four or more MFMAs (128 cycles and up); the two MFMAs of the narrowest tile are over before an LDS read comes back.
+#ifndef TTBFP_AHEAD_MAX_MFMAS
+#define TTBFP_AHEAD_MAX_MFMAS 2
+#endif
+    static constexpr int AHEAD = MB * NB <= TTBFP_AHEAD_MAX_MFMAS ? 2 : 1;
 };
 
 // ---- accumulators ------------------------------------------------------------------------------------
@@ -212,6 +229,24 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v)
     return (uint64_t)lo | ((uint64_t)hi << 32);
 }
 
+// LDS of the ring form: LA A stages, two B stages, LA raw areas (the arithmetic of the kernel's RAW_PITCH)
+template <typename S, int LA>
+constexpr uint32_t ring_lds_bytes()
+{
+    constexpr uint32_t run = (S::BN / kTile) * kW8Tile, cpw = 2 * run / 16 / S::NW, wi = (cpw + 63) / 64;
+    return LA * S::A_BYTES + 2 * S::B_BYTES + LA * (2 * run + (wi * 64 - cpw) * 16);
+}
+
+// LDS of one pipeline: the rings, or two (packed W) or two to three (panel) stages
+template <typename S, bool PANEL, int RING>
+constexpr uint32_t pipeline_lds_bytes()
+{
+    if constexpr (RING > 0)
+        return ring_lds_bytes<S, RING>();
+    else
+        return (PANEL ? panel_stages<S>() : 2) * S::STAGE;
+}
+
 // PANEL: Wp is not the packed weight but its bf16 image made by the panel pre-pass
 // (gemm_bfp8b_panel.hip): for every (column of macro tiles, slab) the B_BYTES of the B stage exactly
 // as the dequantization below would have left them in LDS.  The stage is then filled by direct loads
@@ -228,17 +263,27 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v)
 // anything needs them; the dequantization reads its patch out of the raw area (LDS reads, which the compiler counts apart from
 // loads) into the B stage two iterations ahead as before.  All loads from memory are then direct loads in issue order,
 // and the one wait per iteration names exactly how many of the youngest may stay in flight.
-template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL = false, bool SPLITK = false, int RING = 0>
-__global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t N, uint32_t K, int epilogue,
+//
+// GROUPS = 2: for launches of at most one workgroup per CU on four-wavefront tiles.  A lone wavefront per SIMD issues
+// every instruction of its iteration one behind the other - some 170 per slab for the 128 x 64 tile, against 8 MFMAs - and
+// that, not any unit's throughput, sets its pace.  The workgroup then holds two pipelines of S::NW wavefronts, each with
+// LDS of its own, on the same macro tile: pipeline g multiplies the g-th half of K, and the two meet only at the barriers
+// (both run the same number of iterations) and at the end, where the halves are added through LDS and each pipeline
+// finishes half of the tile's 32 x 32 blocks.  A SIMD then has two wavefronts to issue from.
+template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL = false, bool SPLITK = false, int RING = 0, int GROUPS = 1>
+__global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, uint32_t N, uint32_t K, int epilogue,
                                                            const uint16_t *__restrict__ X,
                                                            const uint8_t *__restrict__ Wp,
                                                            const uint16_t *__restrict__ bias, OutT *__restrict__ Y)
 {
     constexpr int BM = S::BM, BN = S::BN, MB = S::MB, NB = S::NB, XI = S::XI, PW = S::PW, KH = S::KH;
     constexpr uint32_t A_BYTES = S::A_BYTES, STAGE = S::STAGE;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    static_assert(GROUPS == 1 || (GROUPS == 2 && S::NW == 4 && !PANEL && !SPLITK && (MB * NB) % 2 == 0), "two pipelines: packed W, four wavefronts each");
+    const uint32_t group = GROUPS == 1 ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x / S::NT);  // pipeline of this wavefront
+    uint8_t *const lds = lds_all + group * pipeline_lds_bytes<S, PANEL, RING>();
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t tid = threadIdx.x % S::NT, lane = tid & 63;  // thread and wavefront inside the pipeline
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave / S::WN, wn = wave % S::WN;
     // Macro tile of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin and each XCD has
@@ -272,8 +317,8 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     const uint32_t tiles_n = N / kTile;
     static_assert(!(SPLITK && PANEL) && (!SPLITK || sizeof(OutT) == 4), "k split: packed W, fp32 partial sums");
     static_assert(RING == 0 || (RING >= 3 && !PANEL && !SPLITK && S::NW == 4), "rings: three or more stages, packed W, four wavefronts");
-    const uint32_t split = SPLITK ? blockIdx.y : 0;
-    const uint32_t nslabs = SPLITK ? K / BK / gridDim.y : K / BK;  // slabs split * nslabs .. + nslabs - 1
+    const uint32_t split = SPLITK ? blockIdx.y : group;
+    const uint32_t nslabs = SPLITK ? K / BK / gridDim.y : K / BK / GROUPS;  // slabs split * nslabs .. + nslabs - 1
     if constexpr (SPLITK) Y += (uint64_t)split * M * N;
 
     // ---- X: direct loads.  Load i of this wave fills rows (wave XI + i) 8 .. + 7 of the stage; lane l
@@ -309,7 +354,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     const uint32_t w_n = (tid % (BN / PW)) * PW, w_kc = tid / (BN / PW) / (8 / KH), w_half = KH == 8 ? 0 : (tid / (BN / PW)) & 1;
     const uint32_t w_face = ((w_kc >> 1) & 1) * 2 + ((w_n >> 4) & 1), w_kh = w_kc & 1;
     const uint32_t w_in_tile = w_face * 256 + w_kh * 128 + w_half * 64 + (w_n & 15);
-    const uint32_t w_key = ((w_n >> 3) ^ (w_n >> 6)) & 7u;
+    const uint32_t w_key = swizzle_key<KH == 4>(w_n);
     const uint32_t w_lds = A_BYTES + (w_kc * BN + (w_n & ~7u)) * 16 + w_half * 8;  // the 8-column group the patch lies in
     const uint64_t w_slab_bytes = (uint64_t)(BK / kTile) * tiles_n * kW8Tile;
     const uint8_t *w_src = Wp + ((uint64_t)(w_kc >> 2) * tiles_n + n0 / kTile + w_n / kTile) * kW8Tile + (uint64_t)split * nslabs * w_slab_bytes;
@@ -405,7 +450,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         const uint32_t run = cc / (RUN_BYTES / 16), within = cc % (RUN_BYTES / 16);
         raw_off[i] = run * tiles_n * kW8Tile + within * 16;
     }
-    const uint64_t raw_wave = uniform64((uint64_t)(uintptr_t)Wp + (uint64_t)(n0 / kTile) * kW8Tile);
+    const uint64_t raw_wave = uniform64((uint64_t)(uintptr_t)Wp + (uint64_t)(n0 / kTile) * kW8Tile + (uint64_t)split * nslabs * w_slab_bytes);
     auto load_x_ring = [&](uint32_t slab, uint32_t slot, auto ic) {
         constexpr int I = decltype(ic)::value;
         direct_load_16<(I % 4) * 1024>(x_wave + (uint64_t)slab * (BK * 2), x_off[I], lds_base + slot * A_BYTES + (wave * XI + I / 4 * 4) * 8 * A_ROW);
@@ -444,9 +489,14 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     uint32_t b_off[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
-        b_off[nb] = A_BYTES + ((lane >> 5) * BN + swizzle_n(wn * (BN / S::WN) + nb * 32 + (lane & 31))) * 16;
+        b_off[nb] = A_BYTES + ((lane >> 5) * BN + swizzle_n<KH == 4>(wn * (BN / S::WN) + nb * 32 + (lane & 31))) * 16;
 
-    bf16x8 fa[2][MB], fb[2][NB];
+    // Operand buffers: k step j of a slab is multiplied out of buffer j % NBUF, which is filled AHEAD k steps earlier.
+    // A group of MFMA slots (four per iteration) holds the MFMAs of one k step and the operand reads of another:
+    // group G reads k step G of the slab at hand and multiplies k step MUL(G) = (G - AHEAD) mod 4 - of the same slab
+    // when G >= AHEAD, of the slab before (read during the previous iteration) otherwise.
+    constexpr int AHEAD = S::AHEAD, NBUF = 2 * AHEAD;
+    bf16x8 fa[NBUF][MB], fb[NBUF][NB];
     // operand read U (0 .. MB+NB-1) of k step KS into fragment buffer BUF
     // (sta: where the A stage begins; stb: A_BYTES before the B stage - in the two-stage forms both are the stage itself)
     auto read_one2 = [&](const uint8_t *sta, const uint8_t *stb, auto uc, auto ksc, auto bufc) {
@@ -493,7 +543,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     static_assert(X_FIRST + (XI - 1) * X_STEP < SLOTS, "every X load needs a slot");
     static_assert(WU <= SLOTS, "every W fetch needs a slot");
 
-    // One iteration (P = s & 1): k step 3 of slab s, then k steps 0..2 of slab s+1 (stage P^1).
+    // One iteration (P = s & 1): the last AHEAD k steps of slab s, then the first 4 - AHEAD of slab s+1 (stage P^1).
     // With STAGING, slab s+2 is assembled in stage P meanwhile and a barrier publishes it at the end.
     auto iteration = [&](uint32_t s, auto pc, auto stagec) {
         constexpr int P = decltype(pc)::value;
@@ -503,10 +553,10 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         // slab whose W is fetched during this iteration; past the end the last slab is fetched again rather than branching
         const uint32_t w_slab = s + 3 < nslabs ? s + 3 : nslabs - 1;
         static_for<4>([&](auto gc) {
-            constexpr int G = decltype(gc)::value;  // group G: MFMAs of k step (G + 3) % 4, operands of the next k step are read
-            k_step(integral_constant<int, (G + 1) & 1>{}, [&](auto uc) {
+            constexpr int G = decltype(gc)::value;  // group G: MFMAs of k step (G - AHEAD) mod 4, operands of k step G are read
+            k_step(integral_constant<int, ((G + 4 - AHEAD) % 4) % NBUF>{}, [&](auto uc) {
                 constexpr int U = decltype(uc)::value, T = G * MF + U;
-                if constexpr (U < MB + NB) read_frag(cur, uc, integral_constant<int, G>{}, integral_constant<int, G & 1>{});
+                if constexpr (U < MB + NB) read_frag(cur, uc, integral_constant<int, G>{}, integral_constant<int, G % NBUF>{});
                 if constexpr (STAGING) {
                     if constexpr (T < WU) fetch_w(w_slab, integral_constant<int, P ^ 1>{}, integral_constant<int, T>{});
                     if constexpr (T == 0) stage_exponents(pc);
@@ -521,7 +571,7 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         });
         if constexpr (STAGING) {
             wait_direct_loads();
-            __syncthreads();  // stage P is complete; every wave holds the operands of k step 3 of slab s+1
+            __syncthreads();  // stage P is complete; every wave holds the operands of the last AHEAD k steps of slab s+1
         }
     };
 
@@ -534,9 +584,9 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         const uint8_t *cur = lds + cur_stage * STAGE;
         static_for<4>([&](auto gc) {
             constexpr int G = decltype(gc)::value;
-            k_step(integral_constant<int, (G + 1) & 1>{}, [&](auto uc) {
+            k_step(integral_constant<int, ((G + 4 - AHEAD) % 4) % NBUF>{}, [&](auto uc) {
                 constexpr int U = decltype(uc)::value, T = G * MF + U;
-                if constexpr (U < MB + NB) read_frag(cur, uc, integral_constant<int, G>{}, integral_constant<int, G & 1>{});
+                if constexpr (U < MB + NB) read_frag(cur, uc, integral_constant<int, G>{}, integral_constant<int, G % NBUF>{});
                 if constexpr (STAGING) {
                     static_for<XI>([&](auto ic) {
                         if constexpr (1 + decltype(ic)::value == T) load_x(s + NSTAGE, dst_stage, ic);
@@ -572,9 +622,9 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         const uint32_t a_dst = slot_of(s), raw_dst = slot_of(s + 1), raw_src = slot_of(s + 2);
         static_for<4>([&](auto gc) {
             constexpr int G = decltype(gc)::value;
-            k_step(integral_constant<int, (G + 1) & 1>{}, [&](auto uc) {
+            k_step(integral_constant<int, ((G + 4 - AHEAD) % 4) % NBUF>{}, [&](auto uc) {
                 constexpr int U = decltype(uc)::value, T = G * MF + U;
-                if constexpr (U < MB + NB) read_frag2(cur_a, cur_b, uc, integral_constant<int, G>{}, integral_constant<int, G & 1>{});
+                if constexpr (U < MB + NB) read_frag2(cur_a, cur_b, uc, integral_constant<int, G>{}, integral_constant<int, G % NBUF>{});
                 if constexpr (STAGING) {
                     if constexpr (T == 0) static_for<WU>([&](auto fc) { fetch_w_ring(raw_src, fc); });
                     if constexpr (T == RING_FIRST - 1) stage_exponents(integral_constant<int, 0>{});
@@ -620,13 +670,16 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         __syncthreads();
         // raw area 0 is free again: slab LA (the main loop goes on with slab LA + 1 in its first iteration)
         static_for<WI>([&](auto ic) { load_raw(last < LA ? last : LA, 0, ic); });
-        // k steps 0..2 of slab 0; the barrier after them frees B stage 0 for slab 2
+        // the first 4 - AHEAD k steps of slab 0 (all four are read); the barrier after them frees B stage 0 for slab 2
         const uint8_t *b0 = lds + A_RING - A_BYTES;
-        static_for<MB + NB>([&](auto uc) { read_one2(lds, b0, uc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
-        static_for<3>([&](auto gc) {
+        static_for<AHEAD>([&](auto kc) {
+            static_for<MB + NB>([&](auto uc) { read_one2(lds, b0, uc, kc, integral_constant<int, decltype(kc)::value % NBUF>{}); });
+        });
+        static_for<4 - AHEAD>([&](auto gc) {
             constexpr int G = decltype(gc)::value;
-            k_step(integral_constant<int, G & 1>{}, [&](auto uc) {
-                if constexpr (decltype(uc)::value < MB + NB) read_frag2(lds, b0, uc, integral_constant<int, G + 1>{}, integral_constant<int, (G + 1) & 1>{});
+            k_step(integral_constant<int, G % NBUF>{}, [&](auto uc) {
+                if constexpr (decltype(uc)::value < MB + NB)
+                    read_frag2(lds, b0, uc, integral_constant<int, G + AHEAD>{}, integral_constant<int, (G + AHEAD) % NBUF>{});
             });
         });
         __syncthreads();
@@ -664,12 +717,15 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     }
     wait_direct_loads();
     __syncthreads();
-    // k steps 0..2 of slab 0; the barrier after them frees stage 0 for slab 2
-    static_for<MB + NB>([&](auto uc) { read_one(lds, uc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
-    static_for<3>([&](auto gc) {
+    // the first 4 - AHEAD k steps of slab 0 (all four are read); the barrier after them frees stage 0 for slab 2
+    static_for<AHEAD>([&](auto kc) {
+        static_for<MB + NB>([&](auto uc) { read_one(lds, uc, kc, integral_constant<int, decltype(kc)::value % NBUF>{}); });
+    });
+    static_for<4 - AHEAD>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
-        k_step(integral_constant<int, G & 1>{}, [&](auto uc) {
-            if constexpr (decltype(uc)::value < MB + NB) read_frag(lds, uc, integral_constant<int, G + 1>{}, integral_constant<int, (G + 1) & 1>{});
+        k_step(integral_constant<int, G % NBUF>{}, [&](auto uc) {
+            if constexpr (decltype(uc)::value < MB + NB)
+                read_frag(lds, uc, integral_constant<int, G + AHEAD>{}, integral_constant<int, (G + AHEAD) % NBUF>{});
         });
     });
     __syncthreads();
@@ -694,12 +750,29 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     }
     }
     }
-    k_step(P1, [&](auto) {});  // k step 3 of the last slab
+    static_for<AHEAD>([&](auto jc) {  // the last AHEAD k steps of the last slab
+        k_step(integral_constant<int, (4 - AHEAD + decltype(jc)::value) % NBUF>{}, [&](auto) {});
+    });
 
     // D layout of the 32x32 MFMA: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
     accumulator_settle<ALL_AGPRS>();
+    // two pipelines: block BLK is finished by pipeline BLK % 2, which gets the other one's partial sums through LDS
+    // ([block][wavefront][register][lane] floats over the start of the workgroup's LDS, which nobody reads any more)
+    float *const exchange = (float *)lds_all;
+    auto exchange_at = [&](int blk, int r) { return exchange + ((blk * S::NW + wave) * 16 + r) * 64 + lane; };
+    if constexpr (GROUPS == 2) {
+        static_assert(MB * NB * S::NW * 16 * 64 * 4 <= 2 * pipeline_lds_bytes<S, PANEL, RING>(), "the exchange fits the workgroup's LDS");
+        __syncthreads();  // both pipelines have read their last operands
+        static_for<MB * NB>([&](auto bc) {
+            constexpr int BLK = decltype(bc)::value;
+            if ((BLK & 1) != (int)group)
+                static_for<16>([&](auto rc) { *exchange_at(BLK, decltype(rc)::value) = accumulator_read<16 * BLK + decltype(rc)::value, ALL_AGPRS>(); });
+        });
+        __syncthreads();
+    }
     static_for<MB * NB>([&](auto bc) {
         constexpr int BLK = decltype(bc)::value, mb = BLK / NB, nb = BLK % NB;
+        if (GROUPS == 2 && (BLK & 1) != (int)group) return;
         const uint32_t col = n0 + wn * (BN / S::WN) + nb * 32 + (lane & 31);
         const float bv = bias ? load_bias(bias, col, epilogue & kEpilogueBiasF32) : 0.0f;
         const uint32_t row0 = m0 + wm * (BM / S::WM) + mb * 32 + (lane >> 5) * 4;
@@ -707,7 +780,9 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
         static_for<16>([&](auto rc) {
             constexpr int r = decltype(rc)::value;
             constexpr uint32_t rr = (r >> 2) * 8 + (r & 3);  // row inside the block, before the lane's 4-row offset
-            float v = accumulator_read<16 * BLK + r, ALL_AGPRS>() + bv;
+            float v = accumulator_read<16 * BLK + r, ALL_AGPRS>();
+            if constexpr (GROUPS == 2) v += *exchange_at(BLK, r);
+            v += bv;
             v = apply_epilogue(epilogue & kEpilogueMask, v);  // uniform branches
             if constexpr (sizeof(OutT) == 4)
                 yp[(uint64_t)rr * N] = v;
@@ -717,55 +792,50 @@ __global__ __launch_bounds__(S::NT) void gemm_bfp8b_kernel(uint32_t M, uint32_t 
     });
 }
 
-template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL>
+template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL, int GROUPS = 1>
 hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
                        void *y, hipStream_t stream)
 {
-    constexpr uint32_t smem = (PANEL ? panel_stages<S>() : 2) * S::STAGE;
-    auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, PANEL>;
+    constexpr uint32_t smem = GROUPS * pipeline_lds_bytes<S, PANEL, 0>();
+    static_assert(smem <= 160 * 1024, "LDS of a CU");
+    if (GROUPS > 1 && (K / BK) % GROUPS) return hipErrorInvalidValue;
+    auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, PANEL, false, 0, GROUPS>;
     static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (attr != hipSuccess) return attr;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
     const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);  // the walk in eighths: see the kernel
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT * GROUPS), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
     return hipGetLastError();
 }
 
-// LDS of the ring form: LA A stages, two B stages, LA raw areas (the arithmetic of the kernel's RAW_PITCH)
-template <typename S, int LA>
-constexpr uint32_t ring_lds_bytes()
-{
-    constexpr uint32_t run = (S::BN / kTile) * kW8Tile, cpw = 2 * run / 16 / S::NW, wi = (cpw + 63) / 64;
-    return LA * S::A_BYTES + 2 * S::B_BYTES + LA * (2 * run + (wi * 64 - cpw) * 16);
-}
-
-template <typename S, typename OutT, bool XCD_BLOCKS, int LA>
+template <typename S, typename OutT, bool XCD_BLOCKS, int LA, int GROUPS = 1>
 hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
                             void *y, hipStream_t stream)
 {
-    constexpr uint32_t smem = ring_lds_bytes<S, LA>();
+    constexpr uint32_t smem = GROUPS * ring_lds_bytes<S, LA>();
     static_assert(smem <= 160 * 1024, "LDS of a CU");
-    auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, false, false, LA>;
+    if (GROUPS > 1 && (K / BK) % GROUPS) return hipErrorInvalidValue;
+    auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, false, false, LA, GROUPS>;
     static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (attr != hipSuccess) return attr;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
     const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT * GROUPS), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
     return hipGetLastError();
 }
 
-template <typename S, typename OutT, int LA>
+template <typename S, typename OutT, int LA, int GROUPS = 1>
 hipError_t launch_shape_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
                              void *y, hipStream_t stream)
 {
     const uint32_t gm = M / S::BM, gn = N / S::BN;
     if (gm % 4 == 0 && gn % 8 == 0 && ((gm / 4) * (gn / 8)) % 8 == 0)
-        return launch_tile_ring<S, OutT, true, LA>(M, N, K, x, w, bias, epilogue, y, stream);
-    return launch_tile_ring<S, OutT, false, LA>(M, N, K, x, w, bias, epilogue, y, stream);
+        return launch_tile_ring<S, OutT, true, LA, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
+    return launch_tile_ring<S, OutT, false, LA, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
 }
 
 // k split: `splits` workgroups per tile, fp32 partial planes [splits][M][N] at `partials`
@@ -791,15 +861,15 @@ bool fits(uint32_t M, uint32_t N, uint32_t K)
     return M % S::BM == 0 && N % S::BN == 0 && K % BK == 0 && K <= (1u << 24);  // 32-bit X offsets inside a wave's rows
 }
 
-template <typename S, typename OutT, bool PANEL = false>
+template <typename S, typename OutT, bool PANEL = false, int GROUPS = 1>
 hipError_t launch_shape(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
                         void *y, hipStream_t stream)
 {
     // 4 x 8 blocks of tiles per XCD need a whole number of rounds of 8 blocks
     const uint32_t gm = M / S::BM, gn = N / S::BN;
     if (gm % 4 == 0 && gn % 8 == 0 && ((gm / 4) * (gn / 8)) % 8 == 0)
-        return launch_tile<S, OutT, true, PANEL>(M, N, K, x, w, bias, epilogue, y, stream);
-    return launch_tile<S, OutT, false, PANEL>(M, N, K, x, w, bias, epilogue, y, stream);
+        return launch_tile<S, OutT, true, PANEL, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
+    return launch_tile<S, OutT, false, PANEL, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
 }
 
 }  // namespace
@@ -834,6 +904,10 @@ TTBFP_DECLARE_GEMM(slim_f32);
 TTBFP_DECLARE_GEMM(slim_bf16);
 TTBFP_DECLARE_GEMM(ring_slim_f32);  // SlimShape in the ring form
 TTBFP_DECLARE_GEMM(ring_slim_bf16);
+TTBFP_DECLARE_GEMM(duo_slim_f32);  // SlimShape in the ring form, two pipelines per workgroup (K a multiple of 128)
+TTBFP_DECLARE_GEMM(duo_slim_bf16);
+TTBFP_DECLARE_GEMM(duo_small_f32);  // SmallShape on two stages, two pipelines per workgroup
+TTBFP_DECLARE_GEMM(duo_small_bf16);
 TTBFP_DECLARE_GEMM(panel_f32);   // BigShape on a bf16 panel of W instead of the packed tiles
 TTBFP_DECLARE_GEMM(panel_bf16);
 TTBFP_DECLARE_GEMM(panel_small_f32);  // SmallShape on a panel made for 128-wide tiles
@@ -842,6 +916,10 @@ TTBFP_DECLARE_GEMM(panel_small_bf16);
     TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, true>(M, N, K, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_RING_GEMM(NAME, SHAPE, OUT_T, LA)                                                                 \
     TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA>(M, N, K, x, w, bias, epilogue, y, stream); }
+#define TTBFP_DEFINE_DUO_GEMM(NAME, SHAPE, OUT_T, LA)                                                                  \
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA, 2>(M, N, K, x, w, bias, epilogue, y, stream); }
+#define TTBFP_DEFINE_DUO_STAGED_GEMM(NAME, SHAPE, OUT_T)                                                               \
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, false, 2>(M, N, K, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_GEMM(NAME, SHAPE, OUT_T)                                                                          \
     TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T>(M, N, K, x, w, bias, epilogue, y, stream); }
 
