@@ -28,19 +28,21 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # device copy (FETCH_SIZE reads half the KiB actually fetched on this part: factor 2.0; WRITE_SIZE
 # factor 1.0).  Summary: profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES = {
-    "tilize_pack": int((524379.0 * 2.0 + 557066.3) * 1024),      # 1,644,363,981 vs 1,644,167,168 algorithmic
-    "unpack_untilize": int((278609.8 * 2.0 + 1048721.4) * 1024),  # 1,644,483,584
+    # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) x 1024 per launch; the two factors come from the 1 GiB copy in the same runs
+    "tilize_pack": 1644319171,      # 1,644,167,168 algorithmic
+    "unpack_untilize": 1644353513,
     # GEMM kernels, same method: profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt (the forms with a workspace include
-    # their first pass / their reduction)
-    "gemm_8192": 1253119488, "gemm_8192_ws": 1965067980, "gemm_M8192": 344782643, "gemm_M8192_ws": 522035916,
-    "gemm_M512": 56064204, "gemm_M512_ws": 89606553, "gemm_M32": 26591027, "gemm_M64": 28969984, "gemm_M128": 33724211,
+    # their first pass / their reduction; the FFN figures are the sums of its two matmuls)
+    "gemm_8192": 1250014729, "gemm_8192_ws": 1963155888, "gemm_M8192": 344823743, "gemm_M8192_ws": 522078465,
+    "gemm_M512": 55898179, "gemm_M512_ws": 123183197, "gemm_M32": 21359929, "gemm_M64": 23724787, "gemm_M128": 28462679,
+    "ffn": 124175696, "ffn_ws": 168405541,
 }
 
 
 # where the `traffic` figures come from: counter summaries under profiles/, taken with the library built at this commit
 TRAFFIC_SOURCE = {"streaming": "profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt",
                   "gemm": "profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt",
-                  "library_commit": "see the header of each file"}
+                  "library_commit": "e55711d"}  # the counters were read on the library built from this commit
 
 
 def parse():
@@ -367,7 +369,7 @@ def main():
         flops = 2.0 * 3072 * 1024 * 4096 * 2
         tf = flops / (ms * 1e-3) / 1e12
         gemm["config5_bert_large_ffn"] = dict(ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2),
-                                              roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+                                              roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", MEASURED_TRAFFIC_BYTES["ffn"]))
         # the same block with scratch memory on offer: the second matmul (3072 x 1024 x 4096) takes the two-pass form
         ws = torch.empty(max(capi.gemm_workspace_bytes(3072, 4096, 1024), capi.gemm_workspace_bytes(3072, 1024, 4096), 16),
                          dtype=torch.uint8, device=dev)
@@ -380,7 +382,7 @@ def main():
         ms = (None if args.eager_timing else time_launches(ffn_ws, args.steps, args.warmup, torch)) or ms
         tf = flops / (ms * 1e-3) / 1e12
         gemm["config5_bert_large_ffn_with_workspace"] = dict(ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2),
-                                                             roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+                                                             roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", MEASURED_TRAFFIC_BYTES["ffn_ws"]))
 
     # ---- CPU baseline: the oracle on a bounded sample of the same workload ---------------------------
     cpu_baseline = None
