@@ -32,10 +32,10 @@ MEASURED_TRAFFIC_BYTES = {
     "tilize_pack": 1644319171,      # 1,644,167,168 algorithmic
     "unpack_untilize": 1644353513,
     # GEMM kernels, same method: profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt (the forms with a workspace include
-    # their first pass / their reduction; the FFN figures are the sums of its two matmuls)
+    # their first pass; the FFN figure is the sum of its two matmuls)
     "gemm_8192": 1250014729, "gemm_8192_ws": 1963155888, "gemm_M8192": 344823743, "gemm_M8192_ws": 522078465,
-    "gemm_M512": 55898179, "gemm_M512_ws": 123183197, "gemm_M32": 21359929, "gemm_M64": 23724787, "gemm_M128": 28462679,
-    "ffn": 124175696, "ffn_ws": 168405541,
+    "gemm_M512": 55898179, "gemm_M32": 21359929, "gemm_M64": 23724787, "gemm_M128": 28462679,
+    "ffn": 124175696,
 }
 
 
@@ -347,7 +347,9 @@ def main():
         for M in (32, 512, 8192):
             gemm[f"config4_M{M}"] = gemm_case(M, 4096, 4096, 3)
         gemm["config4_M8192_with_workspace"] = gemm_case(8192, 4096, 4096, 3, workspace=True)
-        gemm["config4_M512_with_workspace"] = gemm_case(512, 4096, 4096, 3, workspace=True)
+        # few macro tiles: with a workspace K is split over more workgroups (M = 512 no longer qualifies: its fused form is level)
+        gemm["weights4096_M256"] = gemm_case(256, 4096, 4096, 3)
+        gemm["weights4096_M256_with_workspace"] = gemm_case(256, 4096, 4096, 3, workspace=True)
         for M in (64, 128):  # between the decode-like and the prefill-like case of config 4
             gemm[f"weights4096_M{M}"] = gemm_case(M, 4096, 4096, 3)
 
@@ -370,19 +372,6 @@ def main():
         tf = flops / (ms * 1e-3) / 1e12
         gemm["config5_bert_large_ffn"] = dict(ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2),
                                               roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", MEASURED_TRAFFIC_BYTES["ffn"]))
-        # the same block with scratch memory on offer: the second matmul (3072 x 1024 x 4096) takes the two-pass form
-        ws = torch.empty(max(capi.gemm_workspace_bytes(3072, 4096, 1024), capi.gemm_workspace_bytes(3072, 1024, 4096), 16),
-                         dtype=torch.uint8, device=dev)
-
-        def ffn_ws():
-            capi.gemm_bfp8b(xa, w1, 4096, bias=b1, epilogue=capi.EPILOGUE_GELU, out=h, workspace=ws)
-            capi.gemm_bfp8b(h, w2, 1024, bias=b2, out=y, workspace=ws)
-
-        ms, mn = time_kernel(ffn_ws, args.steps, args.warmup, torch)
-        ms = (None if args.eager_timing else time_launches(ffn_ws, args.steps, args.warmup, torch)) or ms
-        tf = flops / (ms * 1e-3) / 1e12
-        gemm["config5_bert_large_ffn_with_workspace"] = dict(ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2),
-                                                             roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", MEASURED_TRAFFIC_BYTES["ffn_ws"]))
 
     # ---- CPU baseline: the oracle on a bounded sample of the same workload ---------------------------
     cpu_baseline = None

@@ -519,8 +519,8 @@ def test_empty_single_tile_and_ragged_shapes(shape):
             assert np.array_equal(got.view(want_back.dtype), want_back)
 
 
-@pytest.mark.parametrize("shape", [(4096, 3072, 64), (4096, 3072, 320), (4096, 4096, 128), (8192, 4096, 4096), (3072, 1024, 64), (3072, 1024, 448),
-                                   (3072, 1152, 4096)])
+@pytest.mark.parametrize("shape", [(4096, 3072, 64), (4096, 3072, 320), (4096, 4096, 128), (8192, 4096, 4096), (6144, 1024, 64), (6144, 1024, 448),
+                                   (6144, 1152, 4096)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 def test_gemm_with_a_workspace_is_bit_identical(shape, out_dtype):
     """The two-pass form (W converted once into a bf16 panel in the caller's workspace) feeds the MFMAs the same operand
@@ -556,8 +556,8 @@ def test_gemm_with_a_workspace_is_bit_identical(shape, out_dtype):
         assert float((got - ref).norm() / ref.norm()) < 1e-5
 
 
-@pytest.mark.parametrize("shape", [(512, 4096, 4096), (256, 4096, 4096), (256, 1024, 4096), (512, 2048, 2048), (1024, 1024, 4096),
-                                   (256, 512, 1280), (256, 512, 960)])  # the last two: runs of four and of five (an odd number of) slabs
+@pytest.mark.parametrize("shape", [(256, 4096, 4096), (256, 1024, 4096), (1024, 1024, 4096), (512, 1024, 4096), (384, 1024, 8192),
+                                   (256, 512, 2048), (256, 512, 2560)])  # the last two: runs of four and of five (an odd number of) slabs
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 def test_gemm_split_over_k_with_a_workspace(shape, out_dtype):
     """Shapes whose 128 x 128 tiles leave CUs idle: with a workspace K is cut into runs whose fp32 partial tiles are added

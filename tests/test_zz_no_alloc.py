@@ -41,9 +41,9 @@ def test_static_scratch_gemm_matches_the_workspace_form_call_after_call():
     capi.check(capi.lib().ttbfp_init(0))
     limit = capi.lib().ttbfp_static_scratch_bytes()
     assert limit == 64 << 20
-    # (M, N, K): split over K with 32 MiB of partial planes; a smaller split (8 MiB) right after it; a bf16 panel (24 MiB);
+    # (M, N, K): split over K with 16 MiB of partial planes; a smaller split (8 MiB) right after it; a bf16 panel (24 MiB);
     # a shape that uses no workspace at all
-    shapes = [(512, 4096, 4096), (256, 1024, 4096), (4096, 3072, 4096), (128, 1024, 1024)]
+    shapes = [(256, 4096, 4096), (256, 1024, 4096), (4096, 3072, 4096), (128, 1024, 1024)]
     for i, (M, N, K) in enumerate(shapes):
         need = capi.gemm_workspace_bytes(M, N, K)
         say("static scratch gemm", (M, N, K), "workspace bytes", need)

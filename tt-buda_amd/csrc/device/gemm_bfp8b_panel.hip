@@ -21,7 +21,7 @@
 #define TTBFP_PANEL_BIG_MIN_M 4096    // measured: equal at 4096 rows, 6-8 % ahead at 8192
 #endif
 #ifndef TTBFP_PANEL_SMALL_MIN_M
-#define TTBFP_PANEL_SMALL_MIN_M 3072  // measured: ahead at 3072 x 1024 x 4096, behind at 1024 rows
+#define TTBFP_PANEL_SMALL_MIN_M 6144  // measured against the fused forms: 6144 x 1024 x 4096 73 against 80 us, level at 3072 and 4096 rows (4096 x 2048 x 2048 behind)
 #endif
 
 namespace ttbfp {

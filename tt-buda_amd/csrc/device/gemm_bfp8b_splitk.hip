@@ -72,25 +72,33 @@ hipError_t launch_reduce(uint32_t splits, uint64_t quads, uint32_t N, const floa
 
 }  // namespace
 
-// How many ways K is cut: 0 = this form does not apply.  A cost model of the measured pieces, in microseconds: a
-// workgroup of the 128 x 128 MFMA kernel takes 0.735 per 64-k slab alone on its CU and two that share a CU 1.09 per pair
-// of slabs (so up to 512 workgroups are worth having); launch, prologue and epilogue cost 5.5; the second launch 3 plus
-// the partial planes written and read once (s M N 8 bytes at 9 TB/s, most of it out of cache).  Predicted / measured
-// at N = K = 4096: M = 512 fused 52.5 / 52.5, two runs 35.7 / 35.5, four runs 33.4 / 33.6; M = 256 four runs 24.0 / 24.5,
-// eight 24.7 / 25.0; 256 x 4096 x 1024 fused 17.3 / 17.0.  The cut with the shortest prediction wins if it saves 3 us or more.
+// How many ways K is cut: 0 = this form does not apply.  A cost model of the measured pieces, in microseconds.  Launch,
+// prologue and epilogue cost 5.5.  The fused kernel that the shape would get otherwise: the 128 x 64 tile with two pipelines
+// takes 0.80 to 0.97 per pair of 64-k slabs (by how many of the CUs have a workgroup), with one pipeline 0.53 per slab; the
+// 128 x 128 tile with two pipelines 1.25 per pair.  A workgroup of the 128 x 128 kernel of this form takes 0.735 per slab alone on
+// its CU and two that share a CU 1.2 per pair of slabs (so up to 512 workgroups are worth having); the second launch costs 3
+// plus the partial planes written and read once (s M N 8 bytes at 9 TB/s, most of it out of cache).  Predicted / measured:
+// 256 x 4096 x 4096 fused 33.8 / 31.8, four runs 24.0 / 24.9; 1024 x 1024 x 4096 33.8 / 31.3 and 24.0 / 25.7; 256 x 1024 x 4096
+// 31.7 / 29.6, eight runs 16.3 / 17.3; 512 x 4096 x 4096 36.5 / 36.4, four runs 35.2 / 37.3 (not taken); 512 x 2048 x 2048 19.7 / 18.1,
+// four runs 18.1 / 21.2 (not taken).  The cut with the shortest prediction wins if it saves 3 us or more.
 static uint32_t splitk_factor(uint32_t M, uint32_t N, uint32_t K)
 {
     if (!gemm_fits<SmallShape>(M, N, K) || M < 256) return 0;  // up to 255 rows go to the weight-streaming kernel
     const uint64_t tiles = (uint64_t)(M / 128) * (N / 128);
     if (tiles > 256) return 0;
     const uint32_t slabs = K / BK;
+    double fused;
+    if (2 * tiles <= 256)
+        fused = K % 128 == 0 ? 5.5 + (slabs / 2) * (0.80 + 0.17 * (double)(2 * tiles) / 256.0) : 5.5 + slabs * 0.53;
+    else
+        fused = K % 128 == 0 ? 5.5 + (slabs / 2) * 1.25 : 5.5 + slabs * 0.735;
     auto mfma_time = [&](uint32_t s) {
         const uint64_t wgs = tiles * s;
-        const double per_slab = wgs > 256 ? 1.09 : 0.735;  // a pair of workgroups per CU, or one
+        const double per_slab = wgs > 256 ? 1.2 : 0.735;  // a pair of workgroups per CU, or one
         return 5.5 + (double)(slabs / s) * per_slab;
     };
     uint32_t best = 0;
-    double best_time = mfma_time(1) - 3.0;
+    double best_time = fused - 3.0;
     for (uint32_t s = 2; s <= TTBFP_SPLITK_MAX && tiles * s <= 512; ++s) {
         if (slabs % s || slabs / s < 4) continue;
         const double t = mfma_time(s) + 3.0 + (double)s * M * N * 8.0 / 9.0e6;
