@@ -117,8 +117,11 @@ int32_t ttbfp_stream_synchronize(void *stream, int32_t timeout_s);
  * {Float32, Float16_b}; dst in {Bfp8_b, Bfp4_b, Bfp2_b, Float32, Float16_b} (a Float16_b source widens exactly into
  * Float32 tiles through the general kernel: the host layer's full-precision mode, not a conversion of the hot path);
  * a Float16 source goes with dst in {Bfp8, Bfp4, Bfp2, Float16} and with nothing else
- * (pybuda/pybuda/device_connector.py:177-201); RawUInt32 goes to RawUInt32 tiles, a pure permutation
- * of 32-bit elements (the queues of embedding indices: device_connector.py:203-225, 270-277). */
+ * (pybuda/pybuda/device_connector.py:177-201); an integer format goes to tiles of the same format and nothing
+ * else, a pure permutation of its elements: RawUInt32 (the queues of embedding indices: device_connector.py:203-225,
+ * 270-277) and Int32 (int32 tensors, pybuda/pybuda/tensor.py:667-668) of 4-byte elements, RawUInt16 and UInt16 of 2-byte
+ * elements, RawUInt8 and Int8 (int8 tensors, tensor.py:669-670) of single bytes; tile sizes
+ * pybuda/csrc/lower_to_buda/common.cpp:180-186. */
 int32_t ttbfp_tilize_pack(const void *src_dev, uint8_t src_fmt, const uint32_t shape[4],
                           const uint64_t strides_bytes[4], uint8_t dst_fmt, int32_t rounding,
                           void *dst_dev, uint64_t dst_bytes, void *stream);
@@ -126,7 +129,8 @@ int32_t ttbfp_tilize_pack(const void *src_dev, uint8_t src_fmt, const uint32_t s
 /* Tiles in src_fmt -> row-major [w,z,r,c] in dst_fmt (Float32 or Float16_b) with the given byte
  * strides: the conversion inside tt::backend::get_output (backend_api.cpp:700-701).
  * Legal pairs: src in {Bfp8_b, Bfp4_b, Bfp2_b, Float16_b} to either destination;
- * Float32 tiles to Float32 only; src in {Bfp8, Bfp4, Bfp2, Float16} to Float16 only. */
+ * Float32 tiles to Float32 only; src in {Bfp8, Bfp4, Bfp2, Float16} to Float16 only; tiles of an integer format
+ * (see ttbfp_tilize_pack) to row-major elements of the same format only. */
 int32_t ttbfp_unpack_untilize(const void *src_dev, uint8_t src_fmt, const uint32_t shape[4],
                               uint8_t dst_fmt, const uint64_t dst_strides_bytes[4], void *dst_dev,
                               void *stream);

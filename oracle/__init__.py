@@ -16,6 +16,7 @@ _LIB_PATH = os.path.join(_HERE, "libttbfp_oracle.so")
 Float32, Float16_b, Bfp8_b, Bfp4_b, Bfp2_b = 0, 5, 6, 7, 15
 Float16, Bfp8, Bfp4, Bfp2 = 1, 2, 3, 11  # the family with the 5-bit exponent of IEEE half
 RawUInt32 = 0xF2  # integer tensors (embedding indices): tiled as they are
+Int32, UInt16, Int8, RawUInt8, RawUInt16 = 8, 12, 14, 0xF0, 0xF1  # the other integer formats, tiled as they are too
 TRUNCATE, NEAREST = 0, 1
 MANTISSA_BITS = {Bfp8_b: 7, Bfp4_b: 3, Bfp2_b: 1, Bfp8: 7, Bfp4: 3, Bfp2: 1}
 _U32x4 = ctypes.c_uint32 * 4
@@ -97,13 +98,25 @@ def _fmt_of(a):
         return Float16_b
     if a.dtype == np.float16:
         return Float16
-    if a.dtype in (np.uint32, np.int32):
+    if a.dtype == np.uint32:
         return RawUInt32
-    raise TypeError("oracle takes float32, float16 or uint16 (bf16 bit pattern) arrays, got %s" % a.dtype)
+    if a.dtype == np.int32:
+        return Int32
+    if a.dtype == np.int16:
+        return UInt16
+    if a.dtype == np.int8:
+        return Int8
+    if a.dtype == np.uint8:
+        return RawUInt8
+    raise TypeError("oracle takes float32, float16, uint16 (bf16 bit pattern) or integer arrays, got %s" % a.dtype)
+
+
+_INTEGER_ITEMSIZE = {RawUInt32: 4, Int32: 4, RawUInt16: 2, UInt16: 2, RawUInt8: 1, Int8: 1}
 
 
 def _dtype_of(fmt):
-    return {Float32: np.float32, Float16_b: np.uint16, Float16: np.float16, RawUInt32: np.uint32}[fmt]
+    return {Float32: np.float32, Float16_b: np.uint16, Float16: np.float16, RawUInt32: np.uint32, Int32: np.int32, UInt16: np.int16,
+            RawUInt16: np.int16, Int8: np.int8, RawUInt8: np.uint8}[fmt]
 
 
 def _shape4(a):
@@ -185,7 +198,9 @@ def tilize_pack(a, dst_fmt, rounding=TRUNCATE, nthreads=1):
     nbytes = packed_size(dst_fmt, a.shape)
     assert nbytes, "shape must be tile aligned and the format supported"
     out = np.empty(nbytes, dtype=np.uint8)
-    rc = lib().oracle_tilize_pack(_ptr(a), _fmt_of(a), shape, strides, dst_fmt, rounding, _ptr(out), nthreads)
+    # an integer format pairs with itself: the array's item size has to match, its signedness does not matter
+    src_fmt = dst_fmt if dst_fmt in _INTEGER_ITEMSIZE and a.itemsize == _INTEGER_ITEMSIZE[dst_fmt] and a.dtype.kind in "iu" else _fmt_of(a)
+    rc = lib().oracle_tilize_pack(_ptr(a), src_fmt, shape, strides, dst_fmt, rounding, _ptr(out), nthreads)
     assert rc == 0, "oracle_tilize_pack failed"
     return out
 

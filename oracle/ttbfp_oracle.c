@@ -35,8 +35,9 @@ static int is_a_format(int fmt)
 uint32_t oracle_tile_bytes(int fmt)
 {
     switch (fmt) {
-        case ORACLE_FMT_FLOAT32: case ORACLE_FMT_RAW_UINT32: return 4 * TILE_ELEMS;
-        case ORACLE_FMT_FLOAT16_B: case ORACLE_FMT_FLOAT16: return 2 * TILE_ELEMS;
+        case ORACLE_FMT_FLOAT32: case ORACLE_FMT_RAW_UINT32: case ORACLE_FMT_INT32: return 4 * TILE_ELEMS;
+        case ORACLE_FMT_FLOAT16_B: case ORACLE_FMT_FLOAT16: case ORACLE_FMT_RAW_UINT16: case ORACLE_FMT_UINT16: return 2 * TILE_ELEMS;
+        case ORACLE_FMT_RAW_UINT8: case ORACLE_FMT_INT8: return TILE_ELEMS;
         case ORACLE_FMT_BFP8_B: case ORACLE_FMT_BFP8: return TILE_ELEMS + TILE_ELEMS / 16;
         case ORACLE_FMT_BFP4_B: case ORACLE_FMT_BFP4: return TILE_ELEMS / 2 + TILE_ELEMS / 16;
         case ORACLE_FMT_BFP2_B: case ORACLE_FMT_BFP2: return TILE_ELEMS / 4 + TILE_ELEMS / 16;
@@ -44,18 +45,28 @@ uint32_t oracle_tile_bytes(int fmt)
     }
 }
 
-/* RawUInt32 is tiled without conversion, i.e. as Float32 bits are; it pairs with itself only */
+/* The integer formats (pybuda/csrc/lower_to_buda/common.hpp:92-111, sizes common.cpp:180-186) are tiled without
+ * conversion: the 32-bit ones as Float32 bits are, the 16-bit ones as Float16_b bits are, the 8-bit ones as bytes
+ * (ORACLE_FMT_RAW_UINT8 stands for both of them below).  An integer format pairs with itself only. */
+static int is_integer(int f)
+{
+    return f == ORACLE_FMT_RAW_UINT8 || f == ORACLE_FMT_RAW_UINT16 || f == ORACLE_FMT_RAW_UINT32 || f == ORACLE_FMT_INT8 ||
+           f == ORACLE_FMT_UINT16 || f == ORACLE_FMT_INT32;
+}
 static int raw_pair(int *a, int *b)
 {
-    if ((*a == ORACLE_FMT_RAW_UINT32) != (*b == ORACLE_FMT_RAW_UINT32)) return 1;
-    if (*a == ORACLE_FMT_RAW_UINT32) *a = *b = ORACLE_FMT_FLOAT32;
+    if ((is_integer(*a) || is_integer(*b)) && *a != *b) return 1;
+    if (*a == ORACLE_FMT_RAW_UINT32 || *a == ORACLE_FMT_INT32) *a = *b = ORACLE_FMT_FLOAT32;
+    if (*a == ORACLE_FMT_RAW_UINT16 || *a == ORACLE_FMT_UINT16) *a = *b = ORACLE_FMT_FLOAT16_B;
+    if (*a == ORACLE_FMT_INT8) *a = *b = ORACLE_FMT_RAW_UINT8;
     return 0;
 }
 
 static uint32_t plain_itemsize(int fmt)
 {
-    if (fmt == ORACLE_FMT_FLOAT32 || fmt == ORACLE_FMT_RAW_UINT32) return 4;
-    if (fmt == ORACLE_FMT_FLOAT16_B || fmt == ORACLE_FMT_FLOAT16) return 2;
+    if (fmt == ORACLE_FMT_FLOAT32 || fmt == ORACLE_FMT_RAW_UINT32 || fmt == ORACLE_FMT_INT32) return 4;
+    if (fmt == ORACLE_FMT_FLOAT16_B || fmt == ORACLE_FMT_FLOAT16 || fmt == ORACLE_FMT_RAW_UINT16 || fmt == ORACLE_FMT_UINT16) return 2;
+    if (fmt == ORACLE_FMT_RAW_UINT8 || fmt == ORACLE_FMT_INT8) return 1;
     return 0;
 }
 
@@ -381,6 +392,8 @@ int oracle_tilize_pack(const void *src, int src_fmt, const uint32_t shape[4],
             uint64_t tile = (uint64_t)band * tc_n + tc;
             if (is_bfp) {
                 pack_one_tile(gathered, src_fmt, 0, dst_fmt, rounding, (uint8_t *)dst + tile * tb);
+            } else if (isz == 1) { /* bytes: the permutation is all there is */
+                memcpy((uint8_t *)dst + tile * tb, gathered, TILE_ELEMS);
             } else {
                 for (uint32_t i = 0; i < TILE_ELEMS; ++i)
                     convert_plain(load_elem_bits(gathered, src_fmt, i), dst_fmt, rounding, dst,
@@ -415,6 +428,8 @@ int oracle_unpack_untilize(const void *src, int src_fmt, const uint32_t shape[4]
             uint64_t tile = (uint64_t)band * tc_n + tc;
             if (is_bfp) {
                 unpack_one_tile((const uint8_t *)src + tile * tb, src_fmt, dst_fmt, elems, 0);
+            } else if (isz == 1) {
+                memcpy(elems, (const uint8_t *)src + tile * tb, TILE_ELEMS);
             } else {
                 for (uint32_t i = 0; i < TILE_ELEMS; ++i)
                     convert_plain(load_elem_bits(src, src_fmt, tile * TILE_ELEMS + i), dst_fmt,

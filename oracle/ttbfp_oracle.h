@@ -52,7 +52,13 @@ enum {
     ORACLE_FMT_BFP8_B = 6,
     ORACLE_FMT_BFP4_B = 7,
     ORACLE_FMT_BFP2_B = 15,
-    ORACLE_FMT_RAW_UINT32 = 0xF2, /* integer tensors: tiled as they are, pairs with itself only */
+    /* integer tensors: tiled as they are; an integer format pairs with itself only */
+    ORACLE_FMT_INT32 = 8,
+    ORACLE_FMT_UINT16 = 12,
+    ORACLE_FMT_INT8 = 14,
+    ORACLE_FMT_RAW_UINT8 = 0xF0,
+    ORACLE_FMT_RAW_UINT16 = 0xF1,
+    ORACLE_FMT_RAW_UINT32 = 0xF2,
 };
 
 enum { ORACLE_ROUND_TRUNCATE = 0, ORACLE_ROUND_NEAREST = 1 };

@@ -36,7 +36,11 @@ def test_tile_bytes_match_data_format_byte_size():
     assert capi.tile_bytes(F.Bfp2_b) == 320
     # the family with the 5-bit exponent has the same sizes (common.cpp:174-179 does not distinguish)
     assert (capi.tile_bytes(F.Float16), capi.tile_bytes(F.Bfp8), capi.tile_bytes(F.Bfp4), capi.tile_bytes(F.Bfp2)) == (2048, 1088, 576, 320)
-    for unsupported in (4, 8, 9, 10, 12, 14, 0xF0, 0xFF):  # Lf8, integer and raw formats
+    # integer formats: common.cpp:180-186
+    assert (capi.tile_bytes(F.Int32), capi.tile_bytes(F.RawUInt32)) == (4096, 4096)
+    assert (capi.tile_bytes(F.UInt16), capi.tile_bytes(F.RawUInt16)) == (2048, 2048)
+    assert (capi.tile_bytes(F.Int8), capi.tile_bytes(F.RawUInt8)) == (1024, 1024)
+    for unsupported in (4, 9, 10, 13, 0xF3, 0xFF):  # Lf8 and codes that name no format
         assert capi.tile_bytes(unsupported) == 0
 
 

@@ -30,8 +30,14 @@ class DataFormatCode:
     Bfp8 = 2
     Bfp4 = 3
     Bfp2 = 11
-    # integer tensors (embedding indices): tiled as they are, to and from tiles of the same format only
+    # integer tensors (embedding indices as RawUInt32; int32 / int8 tensors as Int32 / Int8): tiled as they are, to and from
+    # tiles of the same format only
     RawUInt32 = 0xF2
+    RawUInt16 = 0xF1
+    RawUInt8 = 0xF0
+    Int32 = 8
+    UInt16 = 12
+    Int8 = 14
 
 
 _U32x4 = ctypes.c_uint32 * 4
@@ -130,8 +136,19 @@ def _stream():
 
 
 _TORCH_FMT = {torch.float32: DataFormatCode.Float32, torch.bfloat16: DataFormatCode.Float16_b,
-              torch.float16: DataFormatCode.Float16, torch.int32: DataFormatCode.RawUInt32}
+              torch.float16: DataFormatCode.Float16, torch.int32: DataFormatCode.RawUInt32, torch.int16: DataFormatCode.UInt16,
+              torch.int8: DataFormatCode.Int8, torch.uint8: DataFormatCode.RawUInt8}
 _FMT_TORCH = {v: k for k, v in _TORCH_FMT.items()}
+_INTEGER_ITEMSIZE = {DataFormatCode.RawUInt32: 4, DataFormatCode.Int32: 4, DataFormatCode.RawUInt16: 2, DataFormatCode.UInt16: 2,
+                     DataFormatCode.RawUInt8: 1, DataFormatCode.Int8: 1}
+
+
+def _fmt_of(tensor, tile_fmt):
+    """Format code of a row-major tensor that goes into / comes out of tiles of ``tile_fmt``: an integer format pairs with
+    itself, so an integer tensor of matching item size takes the tiles' own code, whatever its signedness."""
+    if tile_fmt in _INTEGER_ITEMSIZE and not tensor.dtype.is_floating_point and tensor.element_size() == _INTEGER_ITEMSIZE[tile_fmt]:
+        return tile_fmt
+    return _TORCH_FMT[tensor.dtype]
 
 
 def tile_bytes(fmt):
@@ -153,7 +170,7 @@ def tilize_pack(src, dst_fmt, rounding=ROUND_TRUNCATE, out=None):
     else:
         assert out.is_cuda and out.device == src.device and out.dtype == torch.uint8 and out.is_contiguous(), "out must be a contiguous uint8 device tensor"
     strides = _U64x4(*[s * src.element_size() for s in src.stride()])
-    check(lib().ttbfp_tilize_pack(src.data_ptr(), _TORCH_FMT[src.dtype], _U32x4(*src.shape), strides, dst_fmt, rounding,
+    check(lib().ttbfp_tilize_pack(src.data_ptr(), _fmt_of(src, dst_fmt), _U32x4(*src.shape), strides, dst_fmt, rounding,
                                   out.data_ptr(), out.numel(), _stream()))
     return out
 
@@ -171,7 +188,7 @@ def unpack_untilize(packed, src_fmt, shape, dtype=torch.float32, out=None):
     if packed.numel() < need:
         raise BackendError(RUNTIME_ERROR, f"packed buffer holds {packed.numel()} bytes, {need} needed")
     strides = _U64x4(*[s * out.element_size() for s in out.stride()])
-    check(lib().ttbfp_unpack_untilize(packed.data_ptr(), src_fmt, _U32x4(*shape), _TORCH_FMT[out.dtype], strides,
+    check(lib().ttbfp_unpack_untilize(packed.data_ptr(), src_fmt, _U32x4(*shape), _fmt_of(out, src_fmt), strides,
                                       out.data_ptr(), _stream()))
     return out
 
@@ -198,7 +215,7 @@ def tilize_pack_padded(src, dst_fmt, replicate_rows=False, replicate_cols=False,
     else:
         assert out.is_cuda and out.device == src.device and out.dtype == torch.uint8 and out.is_contiguous()
     strides = _U64x4(*[s * src.element_size() for s in src.stride()])
-    check(lib().ttbfp_tilize_pack_padded(src.data_ptr(), _TORCH_FMT[src.dtype], _U32x4(*src.shape), strides, int(replicate_rows), int(replicate_cols),
+    check(lib().ttbfp_tilize_pack_padded(src.data_ptr(), _fmt_of(src, dst_fmt), _U32x4(*src.shape), strides, int(replicate_rows), int(replicate_cols),
                                          dst_fmt, rounding, ctypes.byref(layout) if layout is not None else None, pitch, out.data_ptr(),
                                          out.numel(), _stream()))
     return out
@@ -223,7 +240,7 @@ def unpack_untilize_narrow(packed, src_fmt, shape, dtype=torch.float32, layout=N
         assert out.is_cuda and out.device == packed.device and tuple(out.shape) == tuple(shape) and out.dtype in _TORCH_FMT
     strides = _U64x4(*[s * out.element_size() for s in out.stride()])
     check(lib().ttbfp_unpack_untilize_narrow(packed.data_ptr(), src_fmt, _U32x4(*shape), ctypes.byref(layout) if layout is not None else None,
-                                             pitch, _TORCH_FMT[out.dtype], strides, out.data_ptr(), _stream()))
+                                             pitch, _fmt_of(out, src_fmt), strides, out.data_ptr(), _stream()))
     return out
 
 
@@ -244,7 +261,7 @@ def tilize_pack_queue(src, dst_fmt, layout, pitch=None, rounding=ROUND_TRUNCATE,
     else:
         assert out.is_cuda and out.device == src.device and out.dtype == torch.uint8 and out.is_contiguous(), "out must be a contiguous uint8 device tensor"
     strides = _U64x4(*[s * src.element_size() for s in src.stride()])
-    check(lib().ttbfp_tilize_pack_queue(src.data_ptr(), _TORCH_FMT[src.dtype], _U32x4(*src.shape), strides, dst_fmt, rounding,
+    check(lib().ttbfp_tilize_pack_queue(src.data_ptr(), _fmt_of(src, dst_fmt), _U32x4(*src.shape), strides, dst_fmt, rounding,
                                         ctypes.byref(layout), pitch, out.data_ptr(), out.numel(), _stream()))
     return out
 
@@ -263,7 +280,7 @@ def unpack_untilize_queue(queue, src_fmt, shape, layout, pitch=None, dtype=torch
         assert out.is_cuda and out.device == queue.device and tuple(out.shape) == tuple(shape) and out.dtype in _TORCH_FMT
     strides = _U64x4(*[s * out.element_size() for s in out.stride()])
     check(lib().ttbfp_unpack_untilize_queue(queue.data_ptr(), src_fmt, _U32x4(*shape), ctypes.byref(layout), pitch,
-                                            _TORCH_FMT[out.dtype], strides, out.data_ptr(), _stream()))
+                                            _fmt_of(out, src_fmt), strides, out.data_ptr(), _stream()))
     return out
 
 

@@ -18,6 +18,10 @@ constexpr uint8_t kFloat32 = 0, kFloat16_b = 5, kBfp8_b = 6, kBfp4_b = 7, kBfp2_
 // the "A" family: 5-bit exponent of IEEE half, shared exponent byte = that exponent padded to 8 bits
 // (docs/public/dataformats.rst:32-41,68)
 constexpr uint8_t kFloat16 = 1, kBfp8 = 2, kBfp4 = 3, kBfp2 = 11;
+// One-byte elements tiled as they are (Int8 and RawUInt8 queues): a tile is 1024 bytes, a face row 16 of them.  The 16-bit
+// and 32-bit integer formats need no code of their own: the Float16_b -> Float16_b and Float32 -> Float32 kernels move
+// bits without looking at them.
+constexpr uint8_t kRaw8 = 0xF0;
 
 __host__ __device__ constexpr int mantissa_bits(uint8_t fmt)
 {
@@ -54,6 +58,7 @@ __device__ __forceinline__ uint32_t f32_pattern_to_half(uint32_t f32_bits)
 __host__ __device__ constexpr uint32_t tile_bytes(uint8_t fmt)
 {
     return fmt == kFloat32     ? 4096u
+           : fmt == kRaw8      ? 1024u
            : fmt == kFloat16_b ? 2048u
            : fmt == kFloat16   ? 2048u
            : mantissa_bits(fmt) == 7 ? 1024u + 64u

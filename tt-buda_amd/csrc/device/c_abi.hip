@@ -58,20 +58,34 @@ int32_t static_scratch(int device, void **out)
     return TTBFP_SUCCESS;
 }
 
-// RawUInt32 (tt::DataFormat 0xF2: integer tensors such as embedding indices, pybuda/pybuda/device_connector.py:270-277)
-// is tiled without any conversion, which is what the Float32 -> Float32 kernels do with the bits they are given.
-constexpr uint8_t kRawUInt32 = 0xF2;
-uint8_t canonical(uint8_t fmt) { return fmt == kRawUInt32 ? (uint8_t)ttbfp::kFloat32 : fmt; }
-// true if the pair is legal as far as raw integers go (raw pairs with raw only); rewrites both to their kernel formats
+// Integer formats (pybuda/csrc/lower_to_buda/common.hpp:92-111; sizes pybuda/csrc/lower_to_buda/common.cpp:180-186): index
+// tensors travel as RawUInt32 (pybuda/pybuda/device_connector.py:270-277), int32 and int8 torch tensors as Int32 and Int8
+// (pybuda/pybuda/tensor.py:667-670).  They are tiled without any conversion: the 32-bit ones by the Float32 -> Float32
+// kernels, which move the bits they are given, the 16-bit ones by the Float16_b -> Float16_b kernels, the 8-bit ones by
+// a byte permutation of their own.  An integer format pairs with itself only.
+constexpr uint8_t kRawUInt8 = 0xF0, kRawUInt16 = 0xF1, kRawUInt32 = 0xF2, kInt32 = 8, kUInt16 = 12, kInt8 = 14;
+bool is_integer(uint8_t fmt) { return fmt == kRawUInt8 || fmt == kRawUInt16 || fmt == kRawUInt32 || fmt == kInt32 || fmt == kUInt16 || fmt == kInt8; }
+uint8_t canonical(uint8_t fmt)
+{
+    switch (fmt) {
+        case kRawUInt32: case kInt32: return ttbfp::kFloat32;
+        case kRawUInt16: case kUInt16: return ttbfp::kFloat16_b;
+        case kRawUInt8: case kInt8: return ttbfp::kRaw8;
+        default: return fmt;
+    }
+}
+// true if the pair is legal as far as integers go (an integer format pairs with itself only); rewrites both to their kernel formats
 bool raw_pair_ok(uint8_t &a, uint8_t &b)
 {
-    if ((a == kRawUInt32) != (b == kRawUInt32)) return false;
+    if ((is_integer(a) || is_integer(b)) && a != b) return false;
     a = canonical(a);
     b = canonical(b);
     return true;
 }
+// bytes per element of a row-major tensor in (kernel) format fmt
+uint32_t plain_itemsize(uint8_t fmt) { return fmt == ttbfp::kFloat32 ? 4 : fmt == ttbfp::kRaw8 ? 1 : 2; }
 
-bool is_plain(uint8_t fmt) { return fmt == ttbfp::kFloat32 || fmt == ttbfp::kFloat16_b || fmt == ttbfp::kFloat16; }
+bool is_plain(uint8_t fmt) { return fmt == ttbfp::kFloat32 || fmt == ttbfp::kFloat16_b || fmt == ttbfp::kFloat16 || fmt == ttbfp::kRaw8; }
 bool is_bfp(uint8_t fmt) { return ttbfp::mantissa_bits(fmt) != 0; }
 
 const char *fmt_name(uint8_t fmt)
@@ -86,6 +100,7 @@ const char *fmt_name(uint8_t fmt)
         case ttbfp::kBfp8: return "Bfp8";
         case ttbfp::kBfp4: return "Bfp4";
         case ttbfp::kBfp2: return "Bfp2";
+        case ttbfp::kRaw8: return "8-bit integer";
         default: return "unsupported";
     }
 }
@@ -249,6 +264,7 @@ int32_t check_pack_formats(const char *fn, uint8_t src_fmt, uint8_t dst_fmt, int
         return fail("%s: source format %u (%s): the source must be Float32, Float16_b or Float16", fn, src_fmt, fmt_name(src_fmt));
     if (!(is_bfp(dst_fmt) || is_plain(dst_fmt)))
         return fail("%s: destination format %u is not one of Bfp8[_b], Bfp4[_b], Bfp2[_b], Float16[_b], Float32", fn, dst_fmt);
+    if ((src_fmt == ttbfp::kRaw8) != (dst_fmt == ttbfp::kRaw8)) return fail("%s: one-byte elements go into one-byte tiles and nothing else does", fn);
     // queues with a 5-bit exponent take IEEE half sources and nothing else does (pybuda/pybuda/device_connector.py:177-201)
     if (ttbfp::is_a_format(dst_fmt) != (src_fmt == ttbfp::kFloat16))
         return fail("%s: %s source with %s destination: Float16 sources go with Float16/Bfp8/Bfp4/Bfp2 only", fn, fmt_name(src_fmt),
@@ -266,6 +282,7 @@ int32_t check_unpack_formats(const char *fn, uint8_t src_fmt, uint8_t dst_fmt)
     if (!is_plain(dst_fmt))
         return fail("%s: destination format %u (%s): the output must be Float32, Float16_b or Float16", fn, dst_fmt,
                     fmt_name(dst_fmt));
+    if ((src_fmt == ttbfp::kRaw8) != (dst_fmt == ttbfp::kRaw8)) return fail("%s: one-byte tiles read back as one-byte elements and nothing else does", fn);
     if (ttbfp::is_a_format(src_fmt) != (dst_fmt == ttbfp::kFloat16))
         return fail("%s: %s tiles read back as %s: Float16/Bfp8/Bfp4/Bfp2 read back as Float16 and nothing else does", fn,
                     fmt_name(src_fmt), fmt_name(dst_fmt));
@@ -314,10 +331,10 @@ int32_t ttbfp_tilize_pack(const void *src_dev, uint8_t src_fmt, const uint32_t s
                           uint64_t dst_bytes, void *stream)
 {
     const char *fn = "ttbfp_tilize_pack";
-    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
     if (int32_t s = check_pack_formats(fn, src_fmt, dst_fmt, rounding)) return s;
     ttbfp::TensorGeom g;
-    if (int32_t s = check_geom(fn, shape, strides_bytes, src_fmt == ttbfp::kFloat32 ? 4 : 2, g)) return s;
+    if (int32_t s = check_geom(fn, shape, strides_bytes, plain_itemsize(src_fmt), g)) return s;
     const uint64_t need = ttbfp_packed_size(dst_fmt, shape);
     if (dst_bytes < need)
         return fail("%s: destination holds %llu bytes, %llu needed", fn, (unsigned long long)dst_bytes,
@@ -332,10 +349,10 @@ int32_t ttbfp_tilize_pack_queue(const void *src_dev, uint8_t src_fmt, const uint
                                 void *dst_dev, uint64_t dst_bytes, void *stream)
 {
     const char *fn = "ttbfp_tilize_pack_queue";
-    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
     if (int32_t s = check_pack_formats(fn, src_fmt, dst_fmt, rounding)) return s;
     ttbfp::TensorGeom g;
-    if (int32_t s = check_geom(fn, shape, strides_bytes, src_fmt == ttbfp::kFloat32 ? 4 : 2, g)) return s;
+    if (int32_t s = check_geom(fn, shape, strides_bytes, plain_itemsize(src_fmt), g)) return s;
     ttbfp::QueueLayout q;
     if (int32_t s = check_layout(fn, dst_fmt, shape, layout, buffer_pitch_bytes, q)) return s;
     const uint64_t per_buffer = ttbfp_queue_buffer_bytes(dst_fmt, shape, layout);
@@ -351,10 +368,10 @@ int32_t ttbfp_unpack_untilize(const void *src_dev, uint8_t src_fmt, const uint32
                               const uint64_t dst_strides_bytes[4], void *dst_dev, void *stream)
 {
     const char *fn = "ttbfp_unpack_untilize";
-    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
     if (int32_t s = check_unpack_formats(fn, src_fmt, dst_fmt)) return s;
     ttbfp::TensorGeom g;
-    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, dst_fmt == ttbfp::kFloat32 ? 4 : 2, g)) return s;
+    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, plain_itemsize(dst_fmt), g)) return s;
     if (ttbfp_packed_size(src_fmt, shape) == 0) return TTBFP_SUCCESS;
     if (!src_dev || !dst_dev) return fail("%s: NULL device pointer", fn);
     return hip_status(ttbfp::launch_unpack_untilize(src_dev, src_fmt, g, dst_fmt, dst_dev, nullptr, (hipStream_t)stream), fn);
@@ -365,10 +382,10 @@ int32_t ttbfp_unpack_untilize_queue(const void *src_dev, uint8_t src_fmt, const 
                                     void *stream)
 {
     const char *fn = "ttbfp_unpack_untilize_queue";
-    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
     if (int32_t s = check_unpack_formats(fn, src_fmt, dst_fmt)) return s;
     ttbfp::TensorGeom g;
-    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, dst_fmt == ttbfp::kFloat32 ? 4 : 2, g)) return s;
+    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, plain_itemsize(dst_fmt), g)) return s;
     ttbfp::QueueLayout q;
     if (int32_t s = check_layout(fn, src_fmt, shape, layout, buffer_pitch_bytes, q)) return s;
     if (ttbfp_queue_buffer_bytes(src_fmt, shape, layout) == 0) return TTBFP_SUCCESS;
@@ -381,11 +398,11 @@ int32_t ttbfp_tilize_pack_padded(const void *src_dev, uint8_t src_fmt, const uin
                                  const ttbfp_queue_layout *layout, uint64_t buffer_pitch_bytes, void *dst_dev, uint64_t dst_bytes, void *stream)
 {
     const char *fn = "ttbfp_tilize_pack_padded";
-    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
     if (int32_t s = check_pack_formats(fn, src_fmt, dst_fmt, rounding)) return s;
     ttbfp::TensorGeom g;
     uint32_t tiled[4];
-    if (int32_t s = check_geom(fn, shape, strides_bytes, src_fmt == ttbfp::kFloat32 ? 4 : 2, g, true, replicate_rows, replicate_cols, tiled)) return s;
+    if (int32_t s = check_geom(fn, shape, strides_bytes, plain_itemsize(src_fmt), g, true, replicate_rows, replicate_cols, tiled)) return s;
     ttbfp::QueueLayout q;
     uint64_t need;
     if (layout) {
@@ -407,11 +424,11 @@ int32_t ttbfp_unpack_untilize_narrow(const void *src_dev, uint8_t src_fmt, const
                                      void *stream)
 {
     const char *fn = "ttbfp_unpack_untilize_narrow";
-    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: RawUInt32 pairs with RawUInt32 only", fn);
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
     if (int32_t s = check_unpack_formats(fn, src_fmt, dst_fmt)) return s;
     ttbfp::TensorGeom g;
     uint32_t tiled[4];
-    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, dst_fmt == ttbfp::kFloat32 ? 4 : 2, g, true, 0, 0, tiled)) return s;
+    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, plain_itemsize(dst_fmt), g, true, 0, 0, tiled)) return s;
     ttbfp::QueueLayout q;
     if (layout) {
         if (int32_t s = check_layout(fn, src_fmt, tiled, layout, buffer_pitch_bytes, q)) return s;

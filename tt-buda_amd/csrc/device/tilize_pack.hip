@@ -278,6 +278,53 @@ __global__ __launch_bounds__(256) void tilize_pack_blocks(const uint8_t *__restr
     }
 }
 
+// One-byte elements (Int8 / RawUInt8 queues): a permutation of bytes, one thread per face row of 16.  Index tensors and
+// quantized constants, a few MB at most: no row kernel.
+template <bool QUEUE>
+__global__ __launch_bounds__(256) void tilize_bytes_blocks(const uint8_t *__restrict__ src, TensorGeom g, uint8_t *__restrict__ dst,
+                                                           uint64_t nblocks, QueueLayout q)
+{
+    constexpr uint32_t TB = tile_bytes(kRaw8);
+    const uint64_t blk = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (blk >= nblocks) return;
+    const uint32_t tiles_c = g.C / kTile, tiles_r = g.R / kTile;
+    const uint32_t face_row = blk % 64;
+    const uint64_t tile = blk / 64;
+    const uint32_t tc = tile % tiles_c;
+    const uint64_t band = tile / tiles_c;
+    const uint32_t tr = band % tiles_r;
+    const uint64_t wz = band / tiles_r;
+    const uint32_t z = wz % g.Z, w = wz / g.Z;
+    const uint32_t face = face_row / kFace, row = face_row % kFace;
+    const uint32_t r = tr * kTile + (face / 2) * kFace + row;
+    const uint32_t c = tc * kTile + (face % 2) * kFace;
+    const bool row_inside = r < g.Rl || g.rep_r;
+    const uint8_t *p = src + w * g.s0 + z * g.s1 + (uint64_t)min(r, g.Rl - 1) * g.s2;
+    uint8_t *tile_out = dst + (QUEUE ? tile_offset(q, w, z, tr, tc) : tile * TB);
+    if constexpr (QUEUE) {
+        if (q.prefix && face_row < 2)  // header (face_row 0) and trailing pad (1) of the slot: zeros
+            for (int k = 0; k < 16; ++k) (face_row ? tile_out + TB : tile_out - 16)[k] = 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const bool inside = row_inside && (c + j < g.Cl || g.rep_c);
+        tile_out[face_row * 16 + j] = inside ? p[(uint64_t)min(c + j, g.Cl - 1) * g.s3] : (uint8_t)0;
+    }
+}
+
+hipError_t launch_bytes(const void *src, const TensorGeom &g, void *dst, const QueueLayout *q, hipStream_t stream)
+{
+    const uint64_t nblocks = (uint64_t)g.W * g.Z * (g.R / kTile) * (g.C / kTile) * 64;
+    if (nblocks == 0) return hipSuccess;
+    const uint64_t grid = (nblocks + 255) / 256;
+    if (grid > 0x7fffffffull) return hipErrorInvalidValue;
+    if (q)
+        hipLaunchKernelGGL(tilize_bytes_blocks<true>, dim3((uint32_t)grid), dim3(256), 0, stream, (const uint8_t *)src, g, (uint8_t *)dst, nblocks, *q);
+    else
+        hipLaunchKernelGGL(tilize_bytes_blocks<false>, dim3((uint32_t)grid), dim3(256), 0, stream, (const uint8_t *)src, g, (uint8_t *)dst, nblocks, QueueLayout{});
+    return hipGetLastError();
+}
+
 // Workgroups per CU of the row kernel.  Each holds 32 KiB of loads in flight, and on tensors of hundreds of MiB three per
 // CU stream faster than the eight that LDS and registers would admit (bf16 [8,1,8192,8192] -> Bfp8_b: 254 against 275 us;
 // fp32 sources 7-8 % likewise); a small grid wants them all, to cover its ramp and its tail.
@@ -366,6 +413,7 @@ hipError_t launch_tilize_pack(const void *src, uint8_t src_fmt, const TensorGeom
         return rounding ? by_format<uint16_t, 1>(dst_fmt, src, g, dst, q, stream)
                         : by_format<uint16_t, 0>(dst_fmt, src, g, dst, q, stream);
     if (src_fmt == kFloat16) return rounding ? by_format_a<1>(dst_fmt, src, g, dst, q, stream) : by_format_a<0>(dst_fmt, src, g, dst, q, stream);
+    if (src_fmt == kRaw8 && dst_fmt == kRaw8) return launch_bytes(src, g, dst, q, stream);
     return hipErrorInvalidValue;
 }
 

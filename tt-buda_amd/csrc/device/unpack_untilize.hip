@@ -204,6 +204,46 @@ __global__ __launch_bounds__(256) void unpack_untilize_blocks(const uint8_t *__r
     }
 }
 
+// One-byte elements (Int8 / RawUInt8 queues): the inverse permutation of bytes, one thread per face row of 16.
+template <bool QUEUE>
+__global__ __launch_bounds__(256) void untilize_bytes_blocks(const uint8_t *__restrict__ src, TensorGeom g, uint8_t *__restrict__ dst,
+                                                             uint64_t nblocks, QueueLayout q)
+{
+    constexpr uint32_t TB = tile_bytes(kRaw8);
+    const uint64_t blk = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (blk >= nblocks) return;
+    const uint32_t tiles_c = g.C / kTile, tiles_r = g.R / kTile;
+    const uint32_t face_row = blk % 64;
+    const uint64_t tile = blk / 64;
+    const uint32_t tc = tile % tiles_c;
+    const uint64_t band = tile / tiles_c;
+    const uint32_t tr = band % tiles_r;
+    const uint64_t wz = band / tiles_r;
+    const uint32_t z = wz % g.Z, w = wz / g.Z;
+    const uint32_t face = face_row / kFace, row = face_row % kFace;
+    const uint32_t r = tr * kTile + (face / 2) * kFace + row;
+    const uint32_t c = tc * kTile + (face % 2) * kFace;
+    if (r >= g.Rl) return;  // narrowed away
+    uint8_t *p = dst + w * g.s0 + z * g.s1 + (uint64_t)r * g.s2 + (uint64_t)c * g.s3;
+    const uint8_t *tile_in = src + (QUEUE ? tile_offset(q, w, z, tr, tc) : tile * TB);
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+        if (c + j < g.Cl) p[j * g.s3] = tile_in[face_row * 16 + j];
+}
+
+hipError_t launch_bytes(const void *src, const TensorGeom &g, void *dst, const QueueLayout *q, hipStream_t stream)
+{
+    const uint64_t nblocks = (uint64_t)g.W * g.Z * (g.R / kTile) * (g.C / kTile) * 64;
+    if (nblocks == 0) return hipSuccess;
+    const uint64_t grid = (nblocks + 255) / 256;
+    if (grid > 0x7fffffffull) return hipErrorInvalidValue;
+    if (q)
+        hipLaunchKernelGGL(untilize_bytes_blocks<true>, dim3((uint32_t)grid), dim3(256), 0, stream, (const uint8_t *)src, g, (uint8_t *)dst, nblocks, *q);
+    else
+        hipLaunchKernelGGL(untilize_bytes_blocks<false>, dim3((uint32_t)grid), dim3(256), 0, stream, (const uint8_t *)src, g, (uint8_t *)dst, nblocks, QueueLayout{});
+    return hipGetLastError();
+}
+
 // Workgroups per CU of the row kernel.  On tensors of hundreds of MiB fewer workgroups in flight than LDS and registers
 // admit stream faster (fewer concurrent streams into HBM), as long as enough bytes stay in flight: a workgroup loads
 // `segment_bytes` of tiles at once and stores 32 KiB.  Measured at 1 GiB of results (us, 8 / 4 / 3 workgroups per CU):
@@ -273,6 +313,7 @@ hipError_t by_format(uint8_t src_fmt, const void *src, const TensorGeom &g, void
 hipError_t launch_unpack_untilize(const void *src, uint8_t src_fmt, const TensorGeom &g, uint8_t dst_fmt, void *dst,
                                   const QueueLayout *q, hipStream_t stream)
 {
+    if (src_fmt == kRaw8 || dst_fmt == kRaw8) return src_fmt == dst_fmt ? launch_bytes(src, g, dst, q, stream) : hipErrorInvalidValue;
     if (dst_fmt == kFloat32) return by_format<float>(src_fmt, src, g, dst, q, stream);
     if (dst_fmt == kFloat16_b) return by_format<uint16_t>(src_fmt, src, g, dst, q, stream);
     if (dst_fmt == kFloat16) {  // the A family reads back as IEEE half, and only the A family does

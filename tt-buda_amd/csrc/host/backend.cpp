@@ -46,10 +46,16 @@ bool a_family(DataFormat f)
 {
     return f == DataFormat::Float16 || f == DataFormat::Bfp8 || f == DataFormat::Bfp4 || f == DataFormat::Bfp2;
 }
+// integer tensors (embedding indices as RawUInt32, int32 / int8 torch tensors as Int32 / Int8: pybuda/pybuda/tensor.py:667-674;
+// device_connector.py:204 also names RawUInt8 and RawUInt16 queues): tiled as they are, an integer format pairs with itself only
+bool integer_format(DataFormat f)
+{
+    return f == DataFormat::RawUInt32 || f == DataFormat::RawUInt16 || f == DataFormat::RawUInt8 || f == DataFormat::Int32 ||
+           f == DataFormat::UInt16 || f == DataFormat::Int8;
+}
 bool queue_format_ok(DataFormat f)
 {
-    return plain_float(f) || a_family(f) || f == DataFormat::Bfp8_b || f == DataFormat::Bfp4_b || f == DataFormat::Bfp2_b ||
-           f == DataFormat::RawUInt32;  // integer tensors (embedding indices), tiled as they are
+    return plain_float(f) || a_family(f) || f == DataFormat::Bfp8_b || f == DataFormat::Bfp4_b || f == DataFormat::Bfp2_b || integer_format(f);
 }
 
 // One stream per calling thread: the boundary is entered concurrently from pusher, feeder and main
@@ -272,7 +278,7 @@ std::uint64_t entry_bytes_of(const tt_dram_io_desc &d, DataFormat storage)
 // keeps fp32 tiles, the family with the 5-bit exponent of IEEE half keeps the halves it is fed, raw integers stay raw.
 DataFormat full_precision_of(DataFormat f)
 {
-    if (f == DataFormat::RawUInt32) return f;
+    if (integer_format(f)) return f;
     return a_family(f) ? DataFormat::Float16 : DataFormat::Float32;
 }
 
@@ -321,9 +327,11 @@ std::uint64_t span_bytes(const tt_PytorchTensorDesc &t)
 DEVICE_STATUS_CODE check_source(const tt_PytorchTensorDesc &t, DataFormat dst, const char *fn)
 {
     if (!t.ptr) return fail(std::string(fn) + ": tensor descriptor has no data pointer");
-    if (t.format == DataFormat::RawUInt32 || dst == DataFormat::RawUInt32) {
-        if (t.format != dst) return fail(std::string(fn) + ": RawUInt32 tensors go with RawUInt32 queues and nothing else does");
-        if (t.itemsize != 4) return fail(std::string(fn) + ": itemsize does not match the format");
+    if (integer_format(t.format) || integer_format(dst)) {
+        if (t.format != dst)
+            return fail(std::string(fn) + ": " + data_format_name(t.format) + " tensor for a " + data_format_name(dst) +
+                        " queue: an integer format goes with queues of the same format and nothing else does");
+        if (t.itemsize != data_format_byte_size(dst)) return fail(std::string(fn) + ": itemsize does not match the format");
         for (int i = 0; i < 4; ++i)
             if (t.shape[i] == 0) return fail(std::string(fn) + ": empty dimension");
         return DEVICE_STATUS_CODE::Success;
@@ -845,7 +853,7 @@ DEVICE_STATUS_CODE get_output(const tt_dram_io_desc &qd, tt_PytorchTensorDesc &o
     // Output formats are the ones pybuda turns back into torch tensors (pybuda/pybuda/tensor.py:730-740):
     // Float32 queues read back as Float32, everything with an 8-bit exponent as Float16_b, unless the
     // caller asked for Float32 by presetting the descriptor's format.
-    DataFormat of = q->storage == DataFormat::RawUInt32 ? DataFormat::RawUInt32
+    DataFormat of = integer_format(q->storage)          ? q->storage
                     : a_family(q->storage)              ? DataFormat::Float16
                     : out.format == DataFormat::Float32 ? DataFormat::Float32
                     : q->storage == DataFormat::Float32 ? DataFormat::Float32

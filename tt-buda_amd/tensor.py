@@ -128,7 +128,10 @@ def pytorch_tensor_to_tensor_desc(t, df: DataFormat = None, element_size=None):
 def tensor_desc_to_pytorch_tensor(desc) -> torch.Tensor:
     """Zero-copy torch view of a descriptor's memory (tensor.py:730-745)."""
     by_format = {DataFormat.Float32: torch.float32, DataFormat.Float16_b: torch.bfloat16,
-                 DataFormat.Float16: torch.float16, DataFormat.RawUInt32: torch.int}
+                 DataFormat.Float16: torch.float16, DataFormat.RawUInt32: torch.int,
+                 # beyond the reference, which reads back RawUInt32 only: the other integer queues, as they were pushed
+                 DataFormat.Int32: torch.int32, DataFormat.Int8: torch.int8, DataFormat.UInt16: torch.int16,
+                 DataFormat.RawUInt16: torch.int16, DataFormat.RawUInt8: torch.uint8}
     if desc.format not in by_format:
         raise RuntimeError(f"Unsupported tensor type({desc.format}) for untilization")
     return torch.frombuffer(desc, dtype=by_format[desc.format]).reshape(list(desc.shape))
