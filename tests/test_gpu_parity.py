@@ -371,13 +371,14 @@ def test_gemm_small_against_the_c_oracle():
 @pytest.mark.parametrize("shape", [(32, 96, 160), (32, 1024, 64), (32, 2048, 64), (32, 3072, 32), (64, 3072, 64), (64, 160, 96), (64, 2080, 32), (96, 1504, 192), (128, 256, 384),
                                    (128, 4096, 4096), (160, 96, 224), (224, 128, 256), (608, 192, 384), (416, 160, 96), (256, 512, 256), (384, 192, 640), (512, 1024, 1024),
                                    (768, 128, 16384), (256, 64, 64), (384, 1088, 192), (128 * 17, 128 * 17, 256), (128, 64, 128), (640, 1600, 192), (1024, 2112, 320), (640, 1600, 384), (2048, 1152, 256),
-                                   (1024, 4096, 128)])
+                                   (1024, 4096, 128), (3072, 4096, 192), (6144, 2048, 64)])
 def test_gemm_kernel_selection_shapes(shape):
     """One shape per kernel path: one to four tile rows (weight streaming; K that splits unevenly over the wavefronts,
     fewer tile rows of W than wavefronts, slices of one, two, three and four whole tile pairs and of odd counts), ragged (general kernel), 128 x 64
     macro tiles (fewer than 256 tiles of 128 x 128; up to 256 of them in the form with rings - one pipeline where K is an odd number of slabs:
     one, three; two pipelines else: one slab each, two, three; N = 64, N a multiple of 64 only - more in the two-stage form: 33 x 8 tiles),
-    128 x 128 macro tiles with two pipelines (16 x 9 and 8 x 32 of them, two slabs and one slab per pipeline), 128 x 128 macro tiles (17 x 17 of them), and
+    128 x 128 macro tiles with two pipelines (16 x 9 and 8 x 32 of them, two slabs and one slab per pipeline), 384 x 128 macro tiles
+    (8 x 32 and 16 x 16 of them, where they fill the CUs better than 256 x 256: three slabs, one slab), 128 x 128 macro tiles (17 x 17 of them), and
     enough tiles for the 256 x 256 macro tiles (M = 768); all against
     dequantize-then-fp32-matmul with bias and GELU in both of the reference's forms."""
     M, K, N = shape

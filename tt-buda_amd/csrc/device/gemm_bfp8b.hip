@@ -36,7 +36,17 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
     const bool f32 = y_fmt == kFloat32;
     // Large problems: 256 x 256 macro tiles (eight wavefronts); smaller ones 128 x 128 so that every CU gets work.
     const uint64_t big_tiles = (uint64_t)(M / 256) * (N / 256);
-    if (gemm_fits<BigShape>(M, N, K) && big_tiles >= TTBFP_BIG_MIN_TILES && force_tile() != 1 && force_tile() != 2)
+    const bool big_ok = gemm_fits<BigShape>(M, N, K) && big_tiles >= TTBFP_BIG_MIN_TILES;
+    // 384 x 128 tiles where they fill the CUs better: a round of them costs 0.84 of a round of 256 x 256 tiles (three quarters
+    // of the area at a higher cost per MFMA: 3072 x 4096 x 1024 36 us against 41 with 192 tiles of 256 x 256; 3072 x 4096 x 4096
+    // 114 / 120; 6144 x 4096 x 1024 72 / 75.5)
+    const uint64_t tall_tiles = (uint64_t)(M / 384) * (N / 128);
+    const auto rounds = [](uint64_t tiles) { return (double)((tiles + TTBFP_CUS - 1) / TTBFP_CUS); };
+    if (gemm_fits<TallShape>(M, N, K) && tall_tiles >= TTBFP_BIG_MIN_TILES && (force_tile() == 0 || force_tile() == 5) &&
+        (force_tile() == 5 || !big_ok || 0.84 * rounds(tall_tiles) < rounds(big_tiles)))
+        return f32 ? launch_gemm_bfp8b_tall_f32(M, N, K, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_tall_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    if (big_ok && force_tile() != 1 && force_tile() != 2 && force_tile() != 5)
         return f32 ? launch_gemm_bfp8b_big_f32(M, N, K, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_big_bf16(M, N, K, x, w, bias, epilogue, y, stream);
     // Fewer tiles than that: which tile and form, by how many workgroups a CU gets.
@@ -45,7 +55,7 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
     //   else at most one 128 x 128 workgroup per CU: that tile on two stages with two pipelines (K a multiple of 128) -
     //     3072 x 1024 x 4096: 44.5 us against 53 for 384 workgroups of 128 x 64, 512 x 8192 x 2048: 29 against 33;
     //   else 128 x 64 on two stages below 256 tiles of 128 x 128 (three workgroups fit a CU), 128 x 128 above.
-    // TTBFP_GEMM_TILE (1: 128 x 64 on two stages, 2: 128 x 128 on two stages, 3: 256 x 256 where it fits) and
+    // TTBFP_GEMM_TILE (1: 128 x 64 on two stages, 2: 128 x 128 on two stages, 3: 256 x 256 where it fits, 5: 384 x 128 where it fits) and
     // TTBFP_GEMM_PIPELINES=1 (no workgroup with two pipelines) are tuning aids for measurements and override this.
     const int force = force_tile();
     static const bool duo = [] { const char *v = getenv("TTBFP_GEMM_PIPELINES"); return !v || atoi(v) != 1; }();

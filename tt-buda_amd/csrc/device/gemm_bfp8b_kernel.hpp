@@ -108,7 +108,7 @@ struct Shape {
     static_assert(NW == 4 || NW == 8, "one or two wavefronts per SIMD");
     static_assert(MB * NB <= 16 && (NW == 4 || MB * NB <= 8), "the accumulators of a SIMD's wavefronts must fit its AGPRs");
     static_assert(PW == 4 || PW == 8, "a thread dequantizes 4 or 8 columns");
-    static_assert(KH == 8 || (KH == 4 && PW == 4 && BN == 64), "a thread dequantizes a whole k chunk, or half of one at four columns of a 64-column stage");
+    static_assert(KH == 8 || (KH == 4 && PW == 4), "a thread dequantizes a whole k chunk, or half of one at four columns");
     static_assert(MB % 2 == 0, "operand addressing assumes an even number of m blocks per wave");
     static_assert(MB + NB <= 2 * MB * NB, "at most two operand reads per MFMA slot");
     // How many k steps ahead of its MFMAs a k step's operands are read from LDS.  One step is time enough where a k step has
@@ -884,6 +884,9 @@ using SmallShape = Shape<128, 128, 2, 2>;
 // Half as wide: twice the workgroups for shapes whose 128 x 128 tiles leave CUs idle, and half the weights to dequantize
 // per workgroup and slab (a thread holds four k of four columns); three of them fit a CU.
 using SlimShape = Shape<128, 64, 2, 2>;
+// Three tile rows of 128 in one: M = 3072 (24 tile rows of 128) at N = 4096 gives 8 x 32 = 256 workgroups, one per CU, where
+// 256 x 256 tiles give 192.  Eight wavefronts, wave tile 192 x 32.
+using TallShape = Shape<384, 128, 2, 4>;
 
 // true if the problem can be cut into macro tiles of shape S
 template <typename S>
@@ -902,6 +905,8 @@ TTBFP_DECLARE_GEMM(small_f32);
 TTBFP_DECLARE_GEMM(small_bf16);
 TTBFP_DECLARE_GEMM(slim_f32);
 TTBFP_DECLARE_GEMM(slim_bf16);
+TTBFP_DECLARE_GEMM(tall_f32);
+TTBFP_DECLARE_GEMM(tall_bf16);
 TTBFP_DECLARE_GEMM(ring_slim_f32);  // SlimShape in the ring form
 TTBFP_DECLARE_GEMM(ring_slim_bf16);
 TTBFP_DECLARE_GEMM(duo_slim_f32);  // SlimShape in the ring form, two pipelines per workgroup (K a multiple of 128)
