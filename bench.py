@@ -293,6 +293,26 @@ def main():
                                                                 roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
         del qmem
 
+    # the general kernels (any strides and alignments, one thread per face row) and the padding / narrowing forms of the row
+    # kernels, on a 256 MiB fp32 tensor: a source whose element stride is 8 bytes (every other column of a wider tensor), and
+    # a ragged [.., 8190, 8168] view packed with zero padding and read back narrowed
+    if not args.gemm_only:
+        wide = torch.randn(1, 1, 8192, 16384, device=dev)
+        strided = wide[:, :, :, ::2]
+        pk = torch.empty(capi.packed_size(F.Bfp8_b, strided.shape), dtype=torch.uint8, device=dev)
+        b = strided.numel() * 4 + pk.numel()
+        ms, _ = time_kernel(lambda: capi.tilize_pack(strided, F.Bfp8_b, out=pk), args.steps, args.warmup, torch)
+        kernels["tilize_pack_fp32_to_bfp8b_general_strided_source"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        ms, _ = time_kernel(lambda: capi.unpack_untilize(pk, F.Bfp8_b, strided.shape, out=strided), args.steps, args.warmup, torch)
+        kernels["unpack_untilize_bfp8b_to_fp32_general_strided_result"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        ragged = wide[:, :, :8190, :8168]
+        b = ragged.numel() * 4 + pk.numel()
+        ms, _ = time_kernel(lambda: capi.tilize_pack_padded(ragged, F.Bfp8_b, out=pk), args.steps, args.warmup, torch)
+        kernels["tilize_pack_fp32_to_bfp8b_padded_8190x8168"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        ms, _ = time_kernel(lambda: capi.unpack_untilize_narrow(pk, F.Bfp8_b, ragged.shape, out=ragged), args.steps, args.warmup, torch)
+        kernels["unpack_untilize_bfp8b_to_fp32_narrowed_8190x8168"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        del wide, strided, ragged, pk
+
     # ---- Bfp8_b-weight GEMM and the FFN block --------------------------------------------------------
     gemm = {}
     if not args.no_gemm:
@@ -352,6 +372,8 @@ def main():
         gemm["weights4096_M256_with_workspace"] = gemm_case(256, 4096, 4096, 3, workspace=True)
         for M in (64, 128):  # between the decode-like and the prefill-like case of config 4
             gemm[f"weights4096_M{M}"] = gemm_case(M, 4096, 4096, 3)
+
+        gemm["general_kernel_M512_N4128"] = gemm_case(512, 4128, 4096, 3)  # N is no multiple of 64: the bounds-checked general kernel
 
         # BERT-large FFN: X [3072,1024]; W1 [1024,4096], W2 [4096,1024]
         w1, w2 = pack_weight(1024, 4096, 51), pack_weight(4096, 1024, 52)

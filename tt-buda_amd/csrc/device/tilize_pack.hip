@@ -232,17 +232,25 @@ __global__ __launch_bounds__(256) void tilize_pack_blocks(const uint8_t *__restr
     const uint8_t *p = src + w * g.s0 + z * g.s1 + (uint64_t)min(r, g.Rl - 1) * g.s2;
     uint32_t bits[16];
     uint16_t raw[16];  // the half itself, for Float16 tiles
+    // strides are multiples of the element size (checked at the boundary); with an aligned base every element is one load,
+    // else it is put together from bytes
+    const bool whole = (uintptr_t)src % sizeof(SrcT) == 0;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
         const bool inside = row_inside && (c + j < g.Cl || g.rep_c);
         const uint8_t *e = p + (uint64_t)min(c + j, g.Cl - 1) * g.s3;
+        uint32_t v;  // the element's bits, in the low 16 or all 32
         if (sizeof(SrcT) == 4)
-            bits[j] = (uint32_t)e[0] | (uint32_t)e[1] << 8 | (uint32_t)e[2] << 16 | (uint32_t)e[3] << 24;
+            v = whole ? *(const uint32_t *)e : (uint32_t)e[0] | (uint32_t)e[1] << 8 | (uint32_t)e[2] << 16 | (uint32_t)e[3] << 24;
+        else
+            v = whole ? (uint32_t) * (const uint16_t *)e : (uint32_t)e[0] | (uint32_t)e[1] << 8;
+        if (sizeof(SrcT) == 4)
+            bits[j] = v;
         else if (std::is_same<SrcT, half_t>::value) {
-            raw[j] = inside ? (uint16_t)((uint32_t)e[0] | (uint32_t)e[1] << 8) : (uint16_t)0;
+            raw[j] = inside ? (uint16_t)v : (uint16_t)0;
             bits[j] = half_to_f32_pattern(raw[j]);
         } else
-            bits[j] = (uint32_t)e[0] << 16 | (uint32_t)e[1] << 24;
+            bits[j] = v << 16;
         if (!inside) bits[j] = 0;
     }
     uint8_t *tile_out = dst + (QUEUE ? tile_offset(q, w, z, tr, tc) : tile * TB);
