@@ -247,6 +247,33 @@ constexpr uint32_t pipeline_lds_bytes()
         return (PANEL ? panel_stages<S>() : 2) * S::STAGE;
 }
 
+// Bytes that the two pipelines of a workgroup exchange their partial sums through (0 with one pipeline)
+template <typename S, int GROUPS>
+constexpr uint32_t exchange_lds_bytes()
+{
+    return GROUPS == 2 ? (uint32_t)(S::MB * S::NB * S::NW * 16 * 64 * 4) : 0u;
+}
+// A Float16_b result leaves through LDS: the wavefronts lay the tile down row-major (16 bytes of padding per row keep the
+// 2-byte stores of the two half-wavefronts, which are four rows apart, on different banks) and the whole workgroup then
+// writes it out in 16-byte pieces, whole 128-byte lines at a time.
+template <typename S>
+constexpr uint32_t kImagePitch = S::BN * 2 + 16;
+// LDS of a workgroup: what its pipelines need during the K loop, or the exchange area plus the image of the result tile
+template <typename S, typename OutT, bool PANEL, int RING, int GROUPS>
+constexpr uint32_t workgroup_lds_bytes()
+{
+    constexpr uint32_t pipes = GROUPS * pipeline_lds_bytes<S, PANEL, RING>();
+    constexpr uint32_t image = sizeof(OutT) == 2 ? exchange_lds_bytes<S, GROUPS>() + S::BM * kImagePitch<S> : 0u;
+    return pipes > image ? pipes : image;
+}
+// Two fp32 values to a pair of bf16, round to nearest even (lo in the lower half)
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi)
+{
+    uint32_t r;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
+
 // PANEL: Wp is not the packed weight but its bf16 image made by the panel pre-pass
 // (gemm_bfp8b_panel.hip): for every (column of macro tiles, slab) the B_BYTES of the B stage exactly
 // as the dequantization below would have left them in LDS.  The stage is then filled by direct loads
@@ -761,7 +788,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     float *const exchange = (float *)lds_all;
     auto exchange_at = [&](int blk, int r) { return exchange + ((blk * S::NW + wave) * 16 + r) * 64 + lane; };
     if constexpr (GROUPS == 2) {
-        static_assert(MB * NB * S::NW * 16 * 64 * 4 <= 2 * pipeline_lds_bytes<S, PANEL, RING>(), "the exchange fits the workgroup's LDS");
+        static_assert(exchange_lds_bytes<S, GROUPS>() <= 2 * pipeline_lds_bytes<S, PANEL, RING>(), "the exchange fits the workgroup's LDS");
         __syncthreads();  // both pipelines have read their last operands
         static_for<MB * NB>([&](auto bc) {
             constexpr int BLK = decltype(bc)::value;
@@ -770,33 +797,62 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         });
         __syncthreads();
     }
+    constexpr bool STAGED = sizeof(OutT) == 2;  // a bf16 result is assembled in LDS and written out in whole lines
+    constexpr uint32_t PITCH = kImagePitch<S>;
+    uint8_t *const image = lds_all + exchange_lds_bytes<S, GROUPS>();
+    if constexpr (STAGED && GROUPS == 1) __syncthreads();  // every wavefront has read its last operands (two pipelines: the barriers above)
+    auto finished = [&](auto bc, auto rc, float bv) {  // element r of block BLK with bias and activation applied
+        constexpr int BLK = decltype(bc)::value, r = decltype(rc)::value;
+        float v = accumulator_read<16 * BLK + r, ALL_AGPRS>();
+        if constexpr (GROUPS == 2) v += *exchange_at(BLK, r);
+        v += bv;
+        return apply_epilogue(epilogue & kEpilogueMask, v);  // uniform branches
+    };
     static_for<MB * NB>([&](auto bc) {
         constexpr int BLK = decltype(bc)::value, mb = BLK / NB, nb = BLK % NB;
         if (GROUPS == 2 && (BLK & 1) != (int)group) return;
-        const uint32_t col = n0 + wn * (BN / S::WN) + nb * 32 + (lane & 31);
-        const float bv = bias ? load_bias(bias, col, epilogue & kEpilogueBiasF32) : 0.0f;
-        const uint32_t row0 = m0 + wm * (BM / S::WM) + mb * 32 + (lane >> 5) * 4;
-        OutT *yp = Y + (uint64_t)row0 * N + col;
-        static_for<16>([&](auto rc) {
-            constexpr int r = decltype(rc)::value;
-            constexpr uint32_t rr = (r >> 2) * 8 + (r & 3);  // row inside the block, before the lane's 4-row offset
-            float v = accumulator_read<16 * BLK + r, ALL_AGPRS>();
-            if constexpr (GROUPS == 2) v += *exchange_at(BLK, r);
-            v += bv;
-            v = apply_epilogue(epilogue & kEpilogueMask, v);  // uniform branches
-            if constexpr (sizeof(OutT) == 4)
-                yp[(uint64_t)rr * N] = v;
-            else
-                yp[(uint64_t)rr * N] = f32_to_bf16_rne(__float_as_uint(v));
-        });
+        const uint32_t col_in_tile = wn * (BN / S::WN) + nb * 32 + (lane & 31);
+        const uint32_t row_in_tile = wm * (BM / S::WM) + mb * 32 + (lane >> 5) * 4;
+        const float bv = bias ? load_bias(bias, n0 + col_in_tile, epilogue & kEpilogueBiasF32) : 0.0f;
+        if constexpr (STAGED) {
+            uint8_t *ip = image + row_in_tile * PITCH + col_in_tile * 2;
+            static_for<8>([&](auto pc) {
+                constexpr int r0 = 2 * decltype(pc)::value, r1 = r0 + 1;
+                constexpr uint32_t rr0 = (r0 >> 2) * 8 + (r0 & 3), rr1 = (r1 >> 2) * 8 + (r1 & 3);  // rows inside the block, before the lane's 4-row offset
+                const uint32_t pair = pack_bf16_rne(finished(bc, integral_constant<int, r0>{}, bv), finished(bc, integral_constant<int, r1>{}, bv));
+                *(uint16_t *)(ip + rr0 * PITCH) = (uint16_t)pair;
+                *(uint16_t *)(ip + rr1 * PITCH) = (uint16_t)(pair >> 16);
+            });
+        } else {
+            OutT *yp = Y + (uint64_t)(m0 + row_in_tile) * N + n0 + col_in_tile;
+            static_for<16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                constexpr uint32_t rr = (r >> 2) * 8 + (r & 3);
+                yp[(uint64_t)rr * N] = finished(bc, rc, bv);
+            });
+        }
     });
+    if constexpr (STAGED) {
+        __syncthreads();
+        constexpr int LPR = BN * 2 / 16;                // lanes per row of the tile: 16 bytes each
+        constexpr int RPP = S::NT * GROUPS / LPR;       // rows per pass of the whole workgroup
+        static_assert(BM % RPP == 0, "whole passes");
+        const uint32_t row = threadIdx.x / LPR, piece = threadIdx.x % LPR;
+        const uint8_t *from = image + row * PITCH + piece * 16;
+        uint8_t *to = (uint8_t *)Y + ((uint64_t)(m0 + row) * N + n0) * 2 + piece * 16;
+        const uint64_t step = (uint64_t)RPP * N * 2;
+        static_for<BM / RPP>([&](auto pc) {
+            constexpr int PASS = decltype(pc)::value;
+            *(uint4 *)(to + PASS * step) = *(const uint4 *)(from + PASS * RPP * PITCH);
+        });
+    }
 }
 
 template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL, int GROUPS = 1>
 hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
                        void *y, hipStream_t stream)
 {
-    constexpr uint32_t smem = GROUPS * pipeline_lds_bytes<S, PANEL, 0>();
+    constexpr uint32_t smem = workgroup_lds_bytes<S, OutT, PANEL, 0, GROUPS>();
     static_assert(smem <= 160 * 1024, "LDS of a CU");
     if (GROUPS > 1 && (K / BK) % GROUPS) return hipErrorInvalidValue;
     auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, PANEL, false, 0, GROUPS>;
@@ -814,7 +870,7 @@ template <typename S, typename OutT, bool XCD_BLOCKS, int LA, int GROUPS = 1>
 hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
                             void *y, hipStream_t stream)
 {
-    constexpr uint32_t smem = GROUPS * ring_lds_bytes<S, LA>();
+    constexpr uint32_t smem = workgroup_lds_bytes<S, OutT, false, LA, GROUPS>();
     static_assert(smem <= 160 * 1024, "LDS of a CU");
     if (GROUPS > 1 && (K / BK) % GROUPS) return hipErrorInvalidValue;
     auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, false, false, LA, GROUPS>;
