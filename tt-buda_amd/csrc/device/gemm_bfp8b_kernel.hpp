@@ -109,7 +109,6 @@ struct Shape {
     static_assert(MB * NB <= 16 && (NW == 4 || MB * NB <= 8), "the accumulators of a SIMD's wavefronts must fit its AGPRs");
     static_assert(PW == 4 || PW == 8, "a thread dequantizes 4 or 8 columns");
     static_assert(KH == 8 || (KH == 4 && PW == 4), "a thread dequantizes a whole k chunk, or half of one at four columns");
-    static_assert(MB % 2 == 0, "operand addressing assumes an even number of m blocks per wave");
     static_assert(MB + NB <= 2 * MB * NB, "at most two operand reads per MFMA slot");
     // How many k steps ahead of its MFMAs a k step's operands are read from LDS.  One step is time enough where a k step has
     // four or more MFMAs (128 cycles and up); the two MFMAs of the narrowest tile are over before an LDS read comes back.
@@ -511,8 +510,10 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     const uint32_t a_row = (wm * (BM / S::WM) + (lane & 31)) * A_ROW;
     const uint32_t a_chunk = (lane >> 5) ^ (lane & 7) ^ ((lane >> 3) & 3);
     uint32_t a_off[4];
+    // (a wavefront whose first 32-row block has an odd index in the tile - odd MB, odd wm - sees the two keys swapped)
+    const uint32_t a_swap = MB % 2 ? 2 * (wm & 1) : 0;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) a_off[v] = a_row + ((a_chunk ^ (2 * v)) * 16);
+    for (int v = 0; v < 4; ++v) a_off[v] = a_row + ((a_chunk ^ (2 * ((v + a_swap) & 3))) * 16);
     uint32_t b_off[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
@@ -941,8 +942,9 @@ using SmallShape = Shape<128, 128, 2, 2>;
 // per workgroup and slab (a thread holds four k of four columns); three of them fit a CU.
 using SlimShape = Shape<128, 64, 2, 2>;
 // Three tile rows of 128 in one: M = 3072 (24 tile rows of 128) at N = 4096 gives 8 x 32 = 256 workgroups, one per CU, where
-// 256 x 256 tiles give 192.  Eight wavefronts, wave tile 192 x 32.
-using TallShape = Shape<384, 128, 2, 4>;
+// 256 x 256 tiles give 192.  Eight wavefronts, wave tile 96 x 64 (five operand reads for the six MFMAs of a k step; as 192 x 32
+// it would be seven: 3072 x 4096 x 4096 94-97 against 98-103 us).
+using TallShape = Shape<384, 128, 4, 2>;
 
 // true if the problem can be cut into macro tiles of shape S
 template <typename S>
