@@ -857,8 +857,7 @@ hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, const void *x, const 
     static_assert(smem <= 160 * 1024, "LDS of a CU");
     if (GROUPS > 1 && (K / BK) % GROUPS) return hipErrorInvalidValue;
     auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, PANEL, false, 0, GROUPS>;
-    static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (attr != hipSuccess) return attr;
+    if (hipError_t e = allow_dynamic_lds(kernel, smem); e != hipSuccess) return e;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
     const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);  // the walk in eighths: see the kernel
@@ -875,8 +874,7 @@ hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, c
     static_assert(smem <= 160 * 1024, "LDS of a CU");
     if (GROUPS > 1 && (K / BK) % GROUPS) return hipErrorInvalidValue;
     auto kernel = gemm_bfp8b_kernel<S, OutT, XCD_BLOCKS, false, false, LA, GROUPS>;
-    static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (attr != hipSuccess) return attr;
+    if (hipError_t e = allow_dynamic_lds(kernel, smem); e != hipSuccess) return e;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
     const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);
@@ -902,8 +900,7 @@ hipError_t launch_tile_splitk(uint32_t M, uint32_t N, uint32_t K, uint32_t split
 {
     constexpr uint32_t smem = 2 * S::STAGE;
     auto kernel = gemm_bfp8b_kernel<S, float, false, false, true>;
-    static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (attr != hipSuccess) return attr;
+    if (hipError_t e = allow_dynamic_lds(kernel, smem); e != hipSuccess) return e;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7fffffffull || splits == 0 || splits > 65535 || (K / BK) % splits) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles, splits), dim3(S::NT), smem, stream, M, N, K, 0, (const uint16_t *)x,

@@ -211,8 +211,7 @@ hipError_t launch(uint32_t N, uint32_t K, const void *x, const void *w, const vo
 {
     constexpr uint32_t smem = Skinny<RT>::kWaves * Skinny<RT>::kRegion;
     auto kernel = gemm_bfp8b_skinny_kernel<RT, EPILOGUE, OutT>;
-    static hipError_t attr = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (attr != hipSuccess) return attr;
+    if (hipError_t e = allow_dynamic_lds(kernel, smem); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(N / kTile * 2), dim3(64 * Skinny<RT>::kWaves), smem, stream, N, K, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, bias_f32, (OutT *)y);
     return hipGetLastError();

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace ttbfp {
 
 // Row-major [W,Z,R,C] tensor view; strides in bytes, outermost first (tt_PytorchTensorDesc,
@@ -22,6 +24,21 @@ struct TensorGeom {
 };
 
 struct QueueLayout;  // queue_layout.hpp
+
+// A kernel that wants more dynamic LDS than the default limit has to say so once per device.  One 64-bit mask per kernel
+// (the function is instantiated per kernel type) remembers the devices that have been told.
+template <typename Kernel>
+hipError_t allow_dynamic_lds(Kernel kernel, uint32_t bytes)
+{
+    static std::atomic<uint64_t> told{0};
+    int device = 0;
+    if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+    const uint64_t bit = device >= 0 && device < 64 ? 1ull << device : 0;
+    if (bit && (told.load(std::memory_order_acquire) & bit)) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes); e != hipSuccess) return e;
+    told.fetch_or(bit, std::memory_order_release);
+    return hipSuccess;
+}
 
 // q == nullptr: header-less tiles in one run, order [w][z][r/32][c/32]; otherwise the tiles sit in
 // the queue buffers q describes.
