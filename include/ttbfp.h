@@ -267,6 +267,23 @@ int32_t ttbfp_gemm_bfp8b_bf16_static(uint32_t M, uint32_t N, uint32_t K, const v
                                      const void *w_dev, const void *bias_dev, int32_t epilogue,
                                      void *y_dev, uint8_t y_fmt, void *stream);
 
+/* ---- host-memory twins ---------------------------------------------------------------------------
+ * The boundary's contract lists a CPU twin of each conversion.  These run the same datum rules as the kernels (one
+ * shared statement, compiled for the host) on tensors in HOST memory, single-threaded, without any device or stream:
+ * for a host that has no GPU at hand (packing the weights of a device image on a build machine, checking a queue dump).
+ * They are separate entry points and nothing else: no device entry point calls them, and a device entry point
+ * without a GPU fails.  Same arguments, checks, legal format pairs and status codes as ttbfp_tilize_pack
+ * (backend_api.cpp:688-693, 704), ttbfp_unpack_untilize (backend_api.cpp:700-701) and ttbfp_gemm_bfp8b_bf16
+ * (pybuda/pybuda/op/eval/buda/matmul.py:233-249), with results equal bit for bit for the conversions and to fp32
+ * rounding for the matmul (sums in k order, erf / tanh of the C library). */
+int32_t ttbfp_tilize_pack_cpu(const void *src_host, uint8_t src_fmt, const uint32_t shape[4],
+                              const uint64_t strides_bytes[4], uint8_t dst_fmt, int32_t rounding,
+                              void *dst_host, uint64_t dst_bytes);
+int32_t ttbfp_unpack_untilize_cpu(const void *src_host, uint8_t src_fmt, const uint32_t shape[4],
+                                  uint8_t dst_fmt, const uint64_t dst_strides_bytes[4], void *dst_host);
+int32_t ttbfp_gemm_bfp8b_bf16_cpu(uint32_t M, uint32_t N, uint32_t K, const void *x_host, const void *w_host,
+                                  const void *bias_host, int32_t epilogue, void *y_host, uint8_t y_fmt);
+
 #ifdef __cplusplus
 }
 #endif

@@ -100,6 +100,11 @@ SYMBOLS = {
     "ttbfp_gemm_bfp8b_bf16_static": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
                                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
                                                       ctypes.c_uint8, ctypes.c_void_p]),
+    "ttbfp_tilize_pack_cpu": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, _U64x4, ctypes.c_uint8, ctypes.c_int32,
+                                               ctypes.c_void_p, ctypes.c_uint64]),
+    "ttbfp_unpack_untilize_cpu": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, ctypes.c_uint8, _U64x4, ctypes.c_void_p]),
+    "ttbfp_gemm_bfp8b_bf16_cpu": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p,
+                                                   ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_uint8]),
 }
 
 _lib = None
@@ -346,4 +351,45 @@ def gemm_f32(x, w, bias=None, epilogue=EPILOGUE_NONE, out=None):
         assert bias.is_cuda and bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()
     check(lib().ttbfp_gemm_f32(M, N, K, x.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None, epilogue,
                                out.data_ptr(), _stream()))
+    return out
+
+
+# ---- host-memory twins: CPU tensors in, CPU tensors out, no device --------------------------------------------------
+
+def tilize_pack_cpu(src, dst_fmt, rounding=ROUND_TRUNCATE):
+    """``tilize_pack`` on a 4-D tensor in host memory (any strides): the library's CPU twin of the conversion."""
+    assert not src.is_cuda and src.dim() == 4
+    if src.dtype not in _TORCH_FMT:
+        raise BackendError(RUNTIME_ERROR, f"unsupported source dtype {src.dtype}")
+    out = torch.empty(packed_size(dst_fmt, src.shape), dtype=torch.uint8)
+    strides = _U64x4(*[s * src.element_size() for s in src.stride()])
+    check(lib().ttbfp_tilize_pack_cpu(src.data_ptr(), _fmt_of(src, dst_fmt), _U32x4(*src.shape), strides, dst_fmt, rounding, out.data_ptr(), out.numel()))
+    return out
+
+
+def unpack_untilize_cpu(packed, src_fmt, shape, dtype=torch.float32):
+    """``unpack_untilize`` on tiles in host memory."""
+    assert not packed.is_cuda and packed.dtype == torch.uint8 and packed.is_contiguous()
+    need = packed_size(src_fmt, shape)
+    if packed.numel() < need:
+        raise BackendError(RUNTIME_ERROR, f"packed buffer holds {packed.numel()} bytes, {need} needed")
+    out = torch.empty(tuple(shape), dtype=dtype)
+    strides = _U64x4(*[s * out.element_size() for s in out.stride()])
+    check(lib().ttbfp_unpack_untilize_cpu(packed.data_ptr(), src_fmt, _U32x4(*shape), _fmt_of(out, src_fmt), strides, out.data_ptr()))
+    return out
+
+
+def gemm_bfp8b_cpu(x, w_packed, N, bias=None, epilogue=EPILOGUE_NONE, out_dtype=torch.bfloat16):
+    """``gemm_bfp8b`` on host memory: dequantize-then-fp32-matmul, the library's CPU twin of the matmul."""
+    assert not x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.is_contiguous()
+    assert not w_packed.is_cuda and w_packed.dtype == torch.uint8 and w_packed.is_contiguous()
+    M, K = x.shape
+    assert w_packed.numel() >= packed_size(DataFormatCode.Bfp8_b, (1, 1, K, N))
+    if bias is not None:
+        assert not bias.is_cuda and bias.is_contiguous() and bias.numel() >= N and bias.dtype in (torch.bfloat16, torch.float32)
+        if bias.dtype == torch.float32:
+            epilogue |= EPILOGUE_BIAS_F32
+    out = torch.empty(M, N, dtype=out_dtype)
+    check(lib().ttbfp_gemm_bfp8b_bf16_cpu(M, N, K, x.data_ptr(), w_packed.data_ptr(), bias.data_ptr() if bias is not None else None, epilogue,
+                                          out.data_ptr(), _TORCH_FMT[out_dtype]))
     return out

@@ -43,15 +43,15 @@ struct half_t {
 // a zero field (zeros, half denormals) gives a signed zero, so the shared-exponent byte is the fp32
 // block exponent minus 112 and the magnitudes are those of the 11-bit significand.
 constexpr uint32_t kHalfExponentRebase = 112;
-__device__ __forceinline__ uint32_t half_to_f32_pattern(uint32_t h)
+__host__ __device__ __forceinline__ uint32_t half_to_f32_pattern(uint32_t h)
 {
     const uint32_t e = (h >> 10) & 0x1fu;
     return ((h & 0x8000u) << 16) | (e ? ((e + kHalfExponentRebase) << 23) | ((h & 0x3ffu) << 13) : 0u);
 }
 // exact for every value the A family produces; beyond the half range the result is infinity
-__device__ __forceinline__ uint32_t f32_pattern_to_half(uint32_t f32_bits)
+__host__ __device__ __forceinline__ uint32_t f32_pattern_to_half(uint32_t f32_bits)
 {
-    return __builtin_bit_cast(uint16_t, (_Float16)__uint_as_float(f32_bits));
+    return __builtin_bit_cast(uint16_t, (_Float16)__builtin_bit_cast(float, f32_bits));
 }
 
 // data_format_byte_size(fmt, 1024): pybuda/csrc/lower_to_buda/common.cpp:167-190
@@ -93,13 +93,13 @@ __device__ __forceinline__ void store_stream(void *p, const uint4 &v)
     __builtin_nontemporal_store(t, (u32x4_t *)p);
 }
 
-__device__ __forceinline__ uint32_t biased_exponent(uint32_t f32_bits) { return (f32_bits >> 23) & 0xffu; }
+__host__ __device__ __forceinline__ uint32_t biased_exponent(uint32_t f32_bits) { return (f32_bits >> 23) & 0xffu; }
 
 // One datum (sign << M | magnitude) of an fp32 bit pattern under the block's shared exponent.
 // Inputs with a zero exponent field have no leading one and quantize to zero; a zero magnitude is
 // stored without its sign.
 template <int M, int ROUNDING>
-__device__ __forceinline__ uint32_t quantize_datum(uint32_t bits, uint32_t shared_exp)
+__host__ __device__ __forceinline__ uint32_t quantize_datum(uint32_t bits, uint32_t shared_exp)
 {
     const uint32_t e = biased_exponent(bits);
     uint32_t sig = (bits & 0x007fffffu) | 0x00800000u;  // explicit leading one: 24 bits
@@ -120,10 +120,10 @@ __device__ __forceinline__ uint32_t quantize_datum(uint32_t bits, uint32_t share
 
 // fp32 bit pattern of a datum: (-1)^s * mag * 2^(E - 127 - (M - 1)), exact (denormals included).
 template <int M>
-__device__ __forceinline__ uint32_t dequantize_datum(uint32_t datum, uint32_t shared_exp)
+__host__ __device__ __forceinline__ uint32_t dequantize_datum(uint32_t datum, uint32_t shared_exp)
 {
     const uint32_t mag = datum & ((1u << M) - 1u);
-    const int p = 31 - __clz((int)mag);  // leading one of the magnitude (unused when mag == 0)
+    const int p = 31 - __builtin_clz(mag ? mag : 1u);  // leading one of the magnitude (unused when mag == 0)
     const int e = (int)shared_exp - (M - 1 - p);
     const uint32_t normal = ((uint32_t)e << 23) | ((mag << (23 - p)) & 0x007fffffu);
     const uint32_t denorm = mag << (shared_exp + 23 - M);
@@ -249,7 +249,7 @@ __device__ __forceinline__ uint32_t dequantize_datum_scaled(uint64_t piece, int 
     return __float_as_uint(fmaf((float)(d & ((1u << M) - 1u)), __uint_as_float(signed_scale), 0.0f));
 }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(uint32_t bits)
+__host__ __device__ __forceinline__ uint16_t f32_to_bf16_rne(uint32_t bits)
 {
     if ((bits & 0x7f800000u) == 0x7f800000u && (bits & 0x007fffffu)) return (uint16_t)((bits >> 16) | 0x0040u);
     return (uint16_t)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);

@@ -544,6 +544,46 @@ int32_t ttbfp_gemm_f32(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, co
     return hip_status(ttbfp::launch_gemm_f32(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, (hipStream_t)stream), fn);
 }
 
+// ---- host-memory twins (cpu_twins.hip): the same argument checks, no device, no stream ----------------------------
+
+int32_t ttbfp_tilize_pack_cpu(const void *src_host, uint8_t src_fmt, const uint32_t shape[4], const uint64_t strides_bytes[4],
+                              uint8_t dst_fmt, int32_t rounding, void *dst_host, uint64_t dst_bytes)
+{
+    const char *fn = "ttbfp_tilize_pack_cpu";
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
+    if (int32_t s = check_pack_formats(fn, src_fmt, dst_fmt, rounding)) return s;
+    ttbfp::TensorGeom g;
+    if (int32_t s = check_geom(fn, shape, strides_bytes, plain_itemsize(src_fmt), g)) return s;
+    const uint64_t need = ttbfp_packed_size(dst_fmt, shape);
+    if (dst_bytes < need) return fail("%s: destination holds %llu bytes, %llu needed", fn, (unsigned long long)dst_bytes, (unsigned long long)need);
+    if (need == 0) return TTBFP_SUCCESS;
+    if (!src_host || !dst_host) return fail("%s: NULL pointer", fn);
+    return ttbfp::cpu_tilize_pack(src_host, src_fmt, g, dst_fmt, rounding, dst_host) ? TTBFP_SUCCESS : fail("%s: unsupported format pair", fn);
+}
+
+int32_t ttbfp_unpack_untilize_cpu(const void *src_host, uint8_t src_fmt, const uint32_t shape[4], uint8_t dst_fmt,
+                                  const uint64_t dst_strides_bytes[4], void *dst_host)
+{
+    const char *fn = "ttbfp_unpack_untilize_cpu";
+    if (!raw_pair_ok(src_fmt, dst_fmt)) return fail("%s: an integer format (Int8, UInt16, Int32, RawUInt8, RawUInt16, RawUInt32) pairs with itself only", fn);
+    if (int32_t s = check_unpack_formats(fn, src_fmt, dst_fmt)) return s;
+    ttbfp::TensorGeom g;
+    if (int32_t s = check_geom(fn, shape, dst_strides_bytes, plain_itemsize(dst_fmt), g)) return s;
+    if (ttbfp_packed_size(src_fmt, shape) == 0) return TTBFP_SUCCESS;
+    if (!src_host || !dst_host) return fail("%s: NULL pointer", fn);
+    return ttbfp::cpu_unpack_untilize(src_host, src_fmt, g, dst_fmt, dst_host) ? TTBFP_SUCCESS : fail("%s: unsupported format pair", fn);
+}
+
+int32_t ttbfp_gemm_bfp8b_bf16_cpu(uint32_t M, uint32_t N, uint32_t K, const void *x_host, const void *w_host, const void *bias_host,
+                                  int32_t epilogue, void *y_host, uint8_t y_fmt)
+{
+    const char *fn = "ttbfp_gemm_bfp8b_bf16_cpu";
+    bool nothing = false;
+    if (int32_t s = check_gemm(fn, M, N, K, x_host, w_host, bias_host, epilogue, y_host, y_fmt, nothing)) return s;
+    if (nothing) return TTBFP_SUCCESS;
+    return ttbfp::cpu_gemm_bfp8b(M, N, K, x_host, w_host, bias_host, epilogue, y_host, y_fmt) ? TTBFP_SUCCESS : fail("%s: failed", fn);
+}
+
 uint64_t ttbfp_static_scratch_bytes(void) { return TTBFP_STATIC_SCRATCH_BYTES; }
 
 int32_t ttbfp_gemm_bfp8b_bf16_static(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, const void *w_dev, const void *bias_dev,

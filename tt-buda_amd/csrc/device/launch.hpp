@@ -57,6 +57,11 @@ hipError_t launch_gemm_bfp8b(uint32_t M, uint32_t N, uint32_t K, const void *x, 
                              int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
 
 // Plain fp32 GEMM on row-major operands with an fp32 bias row: the matmul of the full-precision (unquantized) mode.
+// the same conversions on host memory (cpu_twins.hip): no GPU involved, never called by a device entry point
+bool cpu_tilize_pack(const void *src, uint8_t src_fmt, const TensorGeom &g, uint8_t dst_fmt, int rounding, void *dst);
+bool cpu_unpack_untilize(const void *src, uint8_t src_fmt, const TensorGeom &g, uint8_t dst_fmt, void *dst);
+bool cpu_gemm_bfp8b(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue, void *y, uint8_t y_fmt);
+
 hipError_t launch_gemm_f32(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue, void *y,
                            hipStream_t stream);
 
