@@ -195,6 +195,15 @@ int32_t ttbfp_unpack_untilize_narrow(const void *src_dev, uint8_t src_fmt, const
                                      const ttbfp_queue_layout *layout, uint64_t buffer_pitch_bytes, uint8_t dst_fmt,
                                      const uint64_t dst_strides_bytes[4], void *dst_dev, void *stream);
 
+/* ttbfp_unpack_untilize / _queue / _narrow (layout NULL: header-less tiles in one run; shape need not be tile aligned) for
+ * callers that want the library to check both buffers: src_bytes is what src_dev holds, dst_bytes what dst_dev holds.
+ * The call fails, before anything is launched, when the tiles of `shape` take more than src_bytes or when the strided
+ * result reaches past dst_bytes.  Same conversion as tt::backend::get_output (backend_api.cpp:700-701), whose result
+ * tensor the backend sizes itself; here the caller owns the destination, so its size travels with it. */
+int32_t ttbfp_unpack_untilize_sized(const void *src_dev, uint64_t src_bytes, uint8_t src_fmt, const uint32_t shape[4],
+                                    const ttbfp_queue_layout *layout, uint64_t buffer_pitch_bytes, uint8_t dst_fmt,
+                                    const uint64_t dst_strides_bytes[4], void *dst_dev, uint64_t dst_bytes, void *stream);
+
 /* The prestriding transform that push_input applies when the queue descriptor carries a tt::Stride
  * (backend_api.cpp:392-407; set for the activation of a strided convolution by
  * pybuda/pybuda/ttdevice.py:1437-1444 with xy_offsets = [(x, y) for y in range(s) for x in range(s)]).
@@ -240,6 +249,15 @@ int32_t ttbfp_gemm_bfp8b_bf16_ws(uint32_t M, uint32_t N, uint32_t K, const void 
                                  const void *w_dev, const void *bias_dev, int32_t epilogue,
                                  void *y_dev, uint8_t y_fmt, void *workspace_dev,
                                  uint64_t workspace_bytes, void *stream);
+
+/* ttbfp_gemm_bfp8b_bf16_ws with the size of every buffer stated (the golden matmul, pybuda/pybuda/op/eval/buda/matmul.py:233-249,
+ * gets its sizes from the tensors themselves; a C caller has to say them): fails before anything is launched when x holds
+ * fewer than 2 M K bytes, w fewer than the Bfp8_b tiles of [K, N], the bias (if any) fewer than N values, or y fewer
+ * than M N results in y_fmt.  workspace_dev may be NULL. */
+int32_t ttbfp_gemm_bfp8b_bf16_sized(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, uint64_t x_bytes,
+                                    const void *w_dev, uint64_t w_bytes, const void *bias_dev, uint64_t bias_bytes,
+                                    int32_t epilogue, void *y_dev, uint64_t y_bytes, uint8_t y_fmt, void *workspace_dev,
+                                    uint64_t workspace_bytes, void *stream);
 
 /* Y[M,N] = epilogue(X[M,K] * W[K,N] + bias[N]), all fp32, row-major, contiguous, any M, N, K > 0; epilogue without
  * TTBFP_EPILOGUE_BIAS_F32 (the bias is always fp32).  The golden matmul (pybuda/pybuda/op/eval/buda/matmul.py:233-249) on

@@ -98,3 +98,38 @@ def test_queue_argument_errors_are_reported_without_a_gpu():
     assert st == capi.RUNTIME_ERROR and b"4352 needed" in L.ttbfp_last_error()
     st = L.ttbfp_unpack_untilize_queue(None, 6, shape, None, 2176, 0, strides, None, None)
     assert st == capi.RUNTIME_ERROR and b"layout is NULL" in L.ttbfp_last_error()
+
+
+def test_sized_entry_points_refuse_short_buffers_without_a_gpu():
+    """The entry points that are told the size of every buffer fail before any launch when one is too small."""
+    L = capi.lib()
+    shape = (ctypes.c_uint32 * 4)(1, 1, 64, 64)
+    strides = (ctypes.c_uint64 * 4)(16384, 16384, 256, 4)
+    tiles = 4 * 1088
+    st = L.ttbfp_unpack_untilize_sized(None, tiles - 1, 6, shape, None, 0, 0, strides, None, 16384, None)
+    assert st == capi.RUNTIME_ERROR and b"source holds 4351 bytes" in L.ttbfp_last_error()
+    st = L.ttbfp_unpack_untilize_sized(None, tiles, 6, shape, None, 0, 0, strides, None, 16383, None)
+    assert st == capi.RUNTIME_ERROR and b"reaches 16384" in L.ttbfp_last_error()
+    wide = (ctypes.c_uint64 * 4)(32768, 32768, 512, 4)  # rows 512 bytes apart: the last element ends at 63 * 512 + 256
+    st = L.ttbfp_unpack_untilize_sized(None, tiles, 6, shape, None, 0, 0, wide, None, 63 * 512 + 255, None)
+    assert st == capi.RUNTIME_ERROR and b"reaches 32512" in L.ttbfp_last_error()
+    ragged = (ctypes.c_uint32 * 4)(1, 1, 40, 33)  # tiles cover 64 x 64; the result is 40 rows of 33 floats
+    st = L.ttbfp_unpack_untilize_sized(None, tiles - 1, 6, ragged, None, 0, 0, (ctypes.c_uint64 * 4)(5280, 5280, 132, 4), None, 5280, None)
+    assert st == capi.RUNTIME_ERROR and b"source holds" in L.ttbfp_last_error()
+    # with both sizes right the call gets as far as the pointer check
+    st = L.ttbfp_unpack_untilize_sized(None, tiles, 6, shape, None, 0, 0, strides, None, 16384, None)
+    assert st == capi.RUNTIME_ERROR and b"NULL device pointer" in L.ttbfp_last_error()
+
+    M, N, K = 64, 96, 128
+    w_need = capi.packed_size(capi.DataFormatCode.Bfp8_b, (1, 1, K, N))
+    args = dict(x=M * K * 2, w=w_need, b=N * 2, y=M * N * 2)
+
+    def call(**short):
+        a = dict(args, **short)
+        return L.ttbfp_gemm_bfp8b_bf16_sized(M, N, K, None, a["x"], None, a["w"], ctypes.c_void_p(16), a["b"], 0, None, a["y"], 5, None, 0, None)
+
+    assert call(x=args["x"] - 1) == capi.RUNTIME_ERROR and b"x holds" in L.ttbfp_last_error()
+    assert call(w=w_need - 1) == capi.RUNTIME_ERROR and b"w holds" in L.ttbfp_last_error()
+    assert call(b=N * 2 - 1) == capi.RUNTIME_ERROR and b"bias holds" in L.ttbfp_last_error()
+    assert call(y=args["y"] - 1) == capi.RUNTIME_ERROR and b"y holds" in L.ttbfp_last_error()
+    assert call() == capi.RUNTIME_ERROR and b"NULL device pointer" in L.ttbfp_last_error()

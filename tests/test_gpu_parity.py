@@ -496,6 +496,42 @@ def test_errors_are_status_codes_not_crashes():
     assert ttb.capi.lib().ttbfp_init(0) == capi.SUCCESS
 
 
+def test_sized_entry_points_match_the_plain_ones_and_guard_the_buffers():
+    """ttbfp_unpack_untilize_sized / ttbfp_gemm_bfp8b_bf16_sized run the same launches as the entry points without sizes
+    and refuse a destination that is one element short, leaving it untouched."""
+    say("sized entry points")
+    rng = np.random.default_rng(77)
+    shape = (2, 1, 64, 96)
+    x = to_dev(rng.standard_normal(shape).astype(np.float32))
+    packed = capi.tilize_pack(x, F.Bfp8_b)
+    want = capi.unpack_untilize(packed, F.Bfp8_b, shape, torch.bfloat16)
+    assert torch.equal(capi.unpack_untilize_sized(packed, F.Bfp8_b, shape, torch.bfloat16), want)
+    ragged = (2, 1, 50, 70)
+    assert torch.equal(capi.unpack_untilize_sized(packed, F.Bfp8_b, ragged, torch.bfloat16), want[:, :, :50, :70])
+    lay = capi.QueueLayout(2, 3, 1, 1, 1, 1, 1, 1)
+    qmem = capi.tilize_pack_queue(x, F.Bfp8_b, lay)
+    assert torch.equal(capi.unpack_untilize_sized(qmem, F.Bfp8_b, shape, torch.bfloat16, layout=lay), want)
+    short = torch.zeros(x.numel() - 1, dtype=torch.bfloat16, device=DEV)
+    st = [s * 2 for s in want.stride()]
+    code = capi.lib().ttbfp_unpack_untilize_sized(packed.data_ptr(), packed.numel(), F.Bfp8_b, (capi.ctypes.c_uint32 * 4)(*shape), None, 0,
+                                                  F.Float16_b, (capi.ctypes.c_uint64 * 4)(*st), short.data_ptr(), short.numel() * 2, None)
+    torch.cuda.synchronize()
+    assert code == capi.RUNTIME_ERROR and "destination holds" in capi.lib().ttbfp_last_error().decode() and not short.any()
+    with pytest.raises(capi.BackendError):  # fewer tiles than the shape needs
+        capi.unpack_untilize_sized(packed[:-1], F.Bfp8_b, shape, torch.bfloat16)
+
+    M, K, N = 96, 128, 160
+    wp = capi.tilize_pack(to_dev((rng.standard_normal((1, 1, K, N)) * 0.05).astype(np.float32)), F.Bfp8_b)
+    a = to_dev(rng.standard_normal((M, K)).astype(np.float32)).bfloat16()
+    b = to_dev(rng.standard_normal(N).astype(np.float32)).bfloat16()
+    assert torch.equal(capi.gemm_bfp8b(a, wp, N, bias=b, epilogue=1, sized=True), capi.gemm_bfp8b(a, wp, N, bias=b, epilogue=1))
+    y = torch.zeros(M * N - 1, dtype=torch.bfloat16, device=DEV)
+    code = capi.lib().ttbfp_gemm_bfp8b_bf16_sized(M, N, K, a.data_ptr(), M * K * 2, wp.data_ptr(), wp.numel(), None, 0, 0, y.data_ptr(),
+                                                  y.numel() * 2, F.Float16_b, None, 0, None)
+    torch.cuda.synchronize()
+    assert code == capi.RUNTIME_ERROR and "y holds" in capi.lib().ttbfp_last_error().decode() and not y.any()
+
+
 @pytest.mark.parametrize("shape", [(0, 1, 32, 32), (1, 0, 64, 64), (1, 1, 32, 32), (1, 1, 32, 32 * 17), (1, 1, 32 * 9, 32), (5, 3, 32, 96),
                                    (1, 1, 64, 32 * 129)])
 def test_empty_single_tile_and_ragged_shapes(shape):

@@ -1,7 +1,8 @@
 """The GEMM entry point that allocates nothing (``ttbfp_gemm_bfp8b_bf16_static``): its workspace is a static device
 array inside the library.  It runs the kernels of ``ttbfp_gemm_bfp8b_bf16_ws``, so on the same inputs the two must
 agree bit for bit - checked on calls in a row that share the array (a larger split over K, a smaller one that leaves
-most of the array as the first call filled it, a bf16 panel), with torch's allocator watched for any request."""
+most of the array as the first call filled it, a bf16 panel), with the driver's count of free device memory (which sees
+a hipMalloc made anywhere in the process, the library included) and torch's allocator watched for any request."""
 import ctypes
 import sys
 
@@ -53,12 +54,16 @@ def test_static_scratch_gemm_matches_the_workspace_form_call_after_call():
         for out_dtype, epi, b in ((torch.bfloat16, capi.EPILOGUE_NONE, None), (torch.float32, capi.EPILOGUE_GELU, bias)):
             want = capi.gemm_bfp8b(x, wp, N, bias=b, epilogue=epi, out_dtype=out_dtype, workspace=ws)
             got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+            gemm_static(x, wp, N, b, epi, got)  # warm-up: the kernels' code objects and attributes are set up once
             torch.cuda.synchronize()
             before = torch.cuda.memory_stats()["allocation.all.allocated"]
+            free_before = torch.cuda.mem_get_info()[0]  # hipMemGetInfo: device memory free, whoever allocated the rest
             gemm_static(x, wp, N, b, epi, got)
             gemm_static(x, wp, N, b, epi, got)  # again on the array as the first call left it
-            assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+            free_during = torch.cuda.mem_get_info()[0]  # the calls have been queued, nothing has been freed yet
             torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before == free_during, "device memory was allocated or freed during the calls"
+            assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
             assert torch.equal(got, want), (M, N, K, out_dtype)
 
 

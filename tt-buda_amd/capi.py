@@ -84,6 +84,8 @@ SYMBOLS = {
                                                   ctypes.c_int32, _LAYOUT_P, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
     "ttbfp_unpack_untilize_narrow": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint8, _U32x4, _LAYOUT_P, ctypes.c_uint64,
                                                       ctypes.c_uint8, _U64x4, ctypes.c_void_p, ctypes.c_void_p]),
+    "ttbfp_unpack_untilize_sized": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint8, _U32x4, _LAYOUT_P, ctypes.c_uint64,
+                                                     ctypes.c_uint8, _U64x4, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
     "ttbfp_prestride_shape": (ctypes.c_uint64, [ctypes.c_uint32, _U32x4, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32 * 2)]),
     "ttbfp_prestride": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_uint32, _U32x4, _U64x4, ctypes.c_uint32, ctypes.c_void_p,
                                          ctypes.c_uint64, ctypes.c_void_p]),
@@ -94,6 +96,10 @@ SYMBOLS = {
     "ttbfp_gemm_bfp8b_bf16_ws": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
                                                   ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
                                                   ctypes.c_uint8, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
+    "ttbfp_gemm_bfp8b_bf16_sized": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64,
+                                                     ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int32,
+                                                     ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint8, ctypes.c_void_p, ctypes.c_uint64,
+                                                     ctypes.c_void_p]),
     "ttbfp_gemm_f32": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                         ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]),
     "ttbfp_static_scratch_bytes": (ctypes.c_uint64, []),
@@ -195,6 +201,26 @@ def unpack_untilize(packed, src_fmt, shape, dtype=torch.float32, out=None):
     strides = _U64x4(*[s * out.element_size() for s in out.stride()])
     check(lib().ttbfp_unpack_untilize(packed.data_ptr(), src_fmt, _U32x4(*shape), _fmt_of(out, src_fmt), strides,
                                       out.data_ptr(), _stream()))
+    return out
+
+
+def _bytes_from(t):
+    """Bytes between a tensor's first element and the end of the memory it lives in."""
+    return t.untyped_storage().nbytes() - t.storage_offset() * t.element_size()
+
+
+def unpack_untilize_sized(packed, src_fmt, shape, dtype=torch.float32, layout=None, pitch=None, out=None):
+    """``unpack_untilize`` / ``_queue`` / ``_narrow`` through the entry point that is told how much memory both sides hold
+    and refuses, before any launch, a source too small for the tiles or a destination the strided result would overrun."""
+    assert packed.is_cuda and packed.dtype == torch.uint8 and packed.is_contiguous()
+    if out is None:
+        out = torch.empty(tuple(shape), dtype=dtype, device=packed.device)
+    strides = _U64x4(*[s * out.element_size() for s in out.stride()])
+    if layout is not None and pitch is None:
+        pitch = queue_buffer_bytes(src_fmt, _tiled(shape), layout)
+    check(lib().ttbfp_unpack_untilize_sized(packed.data_ptr(), packed.numel(), src_fmt, _U32x4(*shape),
+                                            ctypes.byref(layout) if layout is not None else None, pitch or 0, _fmt_of(out, src_fmt), strides,
+                                            out.data_ptr(), _bytes_from(out), _stream()))
     return out
 
 
@@ -307,10 +333,10 @@ def gemm_workspace_bytes(M, N, K):
     return lib().ttbfp_gemm_bfp8b_workspace_bytes(M, N, K)
 
 
-def gemm_bfp8b(x, w_packed, N, bias=None, epilogue=EPILOGUE_NONE, out_dtype=torch.bfloat16, out=None, workspace=None):
+def gemm_bfp8b(x, w_packed, N, bias=None, epilogue=EPILOGUE_NONE, out_dtype=torch.bfloat16, out=None, workspace=None, sized=False):
     """Y = epilogue(X @ dequant(W) + bias).  x: [M, K] bf16 device tensor; w_packed: Bfp8_b tiles of W[K, N]; bias: [N] in bf16,
     or in fp32 (the sum of a bias over a weight stack).  ``workspace``: an optional uint8 device tensor of
-    ``gemm_workspace_bytes(M, N, K)`` bytes."""
+    ``gemm_workspace_bytes(M, N, K)`` bytes.  ``sized``: go through the entry point that is told the size of every buffer."""
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.is_contiguous()
     M, K = x.shape
     assert w_packed.is_cuda and w_packed.dtype == torch.uint8 and w_packed.is_contiguous()
@@ -327,6 +353,14 @@ def gemm_bfp8b(x, w_packed, N, bias=None, epilogue=EPILOGUE_NONE, out_dtype=torc
             epilogue |= EPILOGUE_BIAS_F32
     if workspace is not None:
         assert workspace.is_cuda and workspace.dtype == torch.uint8 and workspace.is_contiguous()
+    if sized:
+        check(lib().ttbfp_gemm_bfp8b_bf16_sized(M, N, K, x.data_ptr(), _bytes_from(x), w_packed.data_ptr(), w_packed.numel(),
+                                                bias.data_ptr() if bias is not None else None, _bytes_from(bias) if bias is not None else 0,
+                                                epilogue, out.data_ptr(), _bytes_from(out), _TORCH_FMT[out.dtype],
+                                                workspace.data_ptr() if workspace is not None else None,
+                                                workspace.numel() if workspace is not None else 0, _stream()))
+        return out
+    if workspace is not None:
         check(lib().ttbfp_gemm_bfp8b_bf16_ws(M, N, K, x.data_ptr(), w_packed.data_ptr(),
                                              bias.data_ptr() if bias is not None else None, epilogue, out.data_ptr(),
                                              _TORCH_FMT[out.dtype], workspace.data_ptr(), workspace.numel(), _stream()))

@@ -438,6 +438,40 @@ int32_t ttbfp_unpack_untilize_narrow(const void *src_dev, uint8_t src_fmt, const
     return hip_status(ttbfp::launch_unpack_untilize(src_dev, src_fmt, g, dst_fmt, dst_dev, layout ? &q : nullptr, (hipStream_t)stream), fn);
 }
 
+int32_t ttbfp_unpack_untilize_sized(const void *src_dev, uint64_t src_bytes, uint8_t src_fmt, const uint32_t shape[4],
+                                    const ttbfp_queue_layout *layout, uint64_t buffer_pitch_bytes, uint8_t dst_fmt,
+                                    const uint64_t dst_strides_bytes[4], void *dst_dev, uint64_t dst_bytes, void *stream)
+{
+    const char *fn = "ttbfp_unpack_untilize_sized";
+    if (!shape || !dst_strides_bytes) return fail("%s: shape and strides must not be NULL", fn);
+    if (shape[2] == 0 || shape[3] == 0) return fail("%s: shape [%u,%u,%u,%u]: rows and columns must be at least 1", fn, shape[0], shape[1], shape[2], shape[3]);
+    const uint32_t tiled[4] = {shape[0], shape[1], align_up_tile(shape[2]), align_up_tile(shape[3])};
+    // bytes the tiles take on the source side
+    uint64_t need_src;
+    if (layout) {
+        const uint64_t per_buffer = ttbfp_queue_buffer_bytes(src_fmt, tiled, layout);
+        need_src = per_buffer ? ((uint64_t)layout->grid_r * layout->grid_c - 1) * buffer_pitch_bytes + per_buffer : 0;
+    } else {
+        need_src = ttbfp_packed_size(src_fmt, tiled);
+    }
+    if (src_bytes < need_src)
+        return fail("%s: source holds %llu bytes, the tiles of [%u,%u,%u,%u] take %llu", fn, (unsigned long long)src_bytes, shape[0], shape[1],
+                    shape[2], shape[3], (unsigned long long)need_src);
+    // bytes from the first to one past the last element written on the destination side
+    const uint32_t item = plain_itemsize(dst_fmt);
+    uint64_t last = 0;
+    for (int i = 0; i < 4; ++i) {
+        if (shape[i] == 0) return TTBFP_SUCCESS;  // nothing to write
+        const uint64_t reach = (uint64_t)(shape[i] - 1) * dst_strides_bytes[i];
+        if (shape[i] > 1 && reach / (shape[i] - 1) != dst_strides_bytes[i]) return fail("%s: stride %d overflows", fn, i);
+        if (last + reach < last) return fail("%s: strides overflow", fn);
+        last += reach;
+    }
+    if (item && dst_bytes < last + item)
+        return fail("%s: destination holds %llu bytes, the strided result reaches %llu", fn, (unsigned long long)dst_bytes, (unsigned long long)(last + item));
+    return ttbfp_unpack_untilize_narrow(src_dev, src_fmt, shape, layout, buffer_pitch_bytes, dst_fmt, dst_strides_bytes, dst_dev, stream);
+}
+
 uint64_t ttbfp_prestride_shape(uint32_t itemsize, const uint32_t shape[4], uint32_t stride, uint32_t rows_cols[2])
 {
     if (!shape || !stride || (itemsize != 2 && itemsize != 4)) return 0;
@@ -530,6 +564,22 @@ int32_t ttbfp_gemm_bfp8b_bf16_ws(uint32_t M, uint32_t N, uint32_t K, const void 
     if (!panel)
         return hip_status(ttbfp::launch_gemm_bfp8b_splitk(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, (hipStream_t)stream), fn);
     return hip_status(ttbfp::launch_gemm_bfp8b_panel(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, (hipStream_t)stream), fn);
+}
+
+int32_t ttbfp_gemm_bfp8b_bf16_sized(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, uint64_t x_bytes, const void *w_dev,
+                                    uint64_t w_bytes, const void *bias_dev, uint64_t bias_bytes, int32_t epilogue, void *y_dev,
+                                    uint64_t y_bytes, uint8_t y_fmt, void *workspace_dev, uint64_t workspace_bytes, void *stream)
+{
+    const char *fn = "ttbfp_gemm_bfp8b_bf16_sized";
+    const uint64_t y_item = y_fmt == ttbfp::kFloat32 ? 4 : 2, bias_item = (epilogue & TTBFP_EPILOGUE_BIAS_F32) ? 4 : 2;
+    const uint32_t w_shape[4] = {1, 1, K, N};
+    if (x_bytes < (uint64_t)M * K * 2) return fail("%s: x holds %llu bytes, M x K bf16 values take %llu", fn, (unsigned long long)x_bytes, (unsigned long long)M * K * 2);
+    if (M % 32 == 0 && N % 32 == 0 && K % 32 == 0 && w_bytes < ttbfp_packed_size(TTBFP_FMT_BFP8_B, w_shape))
+        return fail("%s: w holds %llu bytes, the Bfp8_b tiles of [K, N] take %llu", fn, (unsigned long long)w_bytes,
+                    (unsigned long long)ttbfp_packed_size(TTBFP_FMT_BFP8_B, w_shape));
+    if (bias_dev && bias_bytes < (uint64_t)N * bias_item) return fail("%s: bias holds %llu bytes, N values take %llu", fn, (unsigned long long)bias_bytes, (unsigned long long)N * bias_item);
+    if (y_bytes < (uint64_t)M * N * y_item) return fail("%s: y holds %llu bytes, M x N results take %llu", fn, (unsigned long long)y_bytes, (unsigned long long)M * N * y_item);
+    return ttbfp_gemm_bfp8b_bf16_ws(M, N, K, x_dev, w_dev, bias_dev, epilogue, y_dev, y_fmt, workspace_dev, workspace_bytes, stream);
 }
 
 int32_t ttbfp_gemm_f32(uint32_t M, uint32_t N, uint32_t K, const void *x_dev, const void *w_dev, const void *bias_dev, int32_t epilogue,

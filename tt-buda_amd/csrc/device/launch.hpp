@@ -25,19 +25,42 @@ struct TensorGeom {
 
 struct QueueLayout;  // queue_layout.hpp
 
-// A kernel that wants more dynamic LDS than the default limit has to say so once per device.  One 64-bit mask per kernel
-// (the function is instantiated per kernel type) remembers the devices that have been told.
-template <typename Kernel>
-hipError_t allow_dynamic_lds(Kernel kernel, uint32_t bytes)
+// A kernel that wants more dynamic LDS than the default limit has to say so once per device.  Kernels of one
+// signature share a function-pointer type, so the memory of who has been told is keyed by the kernel's address, not by
+// its type: a small open-addressed table (the library has a few dozen such kernels), one 64-bit device mask per entry.
+// Lock-free; a slot whose key is being claimed by another thread is simply told again, which is harmless.
+struct DynamicLdsTold {
+    static constexpr int kSlots = 256;
+    std::atomic<const void *> key[kSlots];
+    std::atomic<uint64_t> mask[kSlots];
+};
+inline DynamicLdsTold g_dynamic_lds_told{};
+
+inline hipError_t allow_dynamic_lds_at(const void *kernel, uint32_t bytes)
 {
-    static std::atomic<uint64_t> told{0};
     int device = 0;
     if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
     const uint64_t bit = device >= 0 && device < 64 ? 1ull << device : 0;
-    if (bit && (told.load(std::memory_order_acquire) & bit)) return hipSuccess;
-    if (hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes); e != hipSuccess) return e;
-    told.fetch_or(bit, std::memory_order_release);
+    DynamicLdsTold &t = g_dynamic_lds_told;
+    int slot = -1;
+    for (int i = 0, h = (int)(((uintptr_t)kernel >> 4) % DynamicLdsTold::kSlots); i < DynamicLdsTold::kSlots; ++i, h = (h + 1) % DynamicLdsTold::kSlots) {
+        const void *k = t.key[h].load(std::memory_order_acquire);
+        if (k == nullptr) {
+            const void *expected = nullptr;
+            if (t.key[h].compare_exchange_strong(expected, kernel, std::memory_order_acq_rel)) k = kernel;
+            else k = expected;
+        }
+        if (k == kernel) { slot = h; break; }
+    }
+    if (slot >= 0 && bit && (t.mask[slot].load(std::memory_order_acquire) & bit)) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes); e != hipSuccess) return e;
+    if (slot >= 0) t.mask[slot].fetch_or(bit, std::memory_order_release);
     return hipSuccess;
+}
+template <typename Kernel>
+hipError_t allow_dynamic_lds(Kernel kernel, uint32_t bytes)
+{
+    return allow_dynamic_lds_at((const void *)kernel, bytes);
 }
 
 // q == nullptr: header-less tiles in one run, order [w][z][r/32][c/32]; otherwise the tiles sit in

@@ -241,6 +241,8 @@ struct Queue {
     std::uint32_t reserved = 0;                   // entries being written, behind wr + count
     std::uint64_t ticket_next = 0, ticket_done = 0;  // reservations handed out / published
     std::uint32_t readers = 0;                    // get_output calls reading entries right now
+    bool consuming = false;                       // a run_matmul owns the oldest entry: it reads it and then pops it
+    std::vector<std::uint8_t> poisoned;           // per slot: published without having been written (a push failed)
     std::uint32_t in_flight = 0, max_in_flight = 0;  // conversions running outside the lock, and the most there ever were
     std::uint8_t *slot(std::uint32_t s) const { return base + s * entry_bytes; }  // in buffer 0; the others `pitch` apart
     std::uint64_t span(std::uint32_t entries) const { return (buffers - 1) * pitch + entries * entry_bytes; }
@@ -390,6 +392,7 @@ DEVICE_STATUS_CODE reserve_write(Queue &q, std::uint32_t n, int timeout_s, int r
         r.slot0 = (q.wr + q.reserved) % q.slots;
         r.ticket = q.ticket_next++;
         q.reserved += n;
+        for (std::uint32_t i = 0; i < n; ++i) q.poisoned[(r.slot0 + i) % q.slots] = 0;
     } else {
         r.slot0 = ram_ptr < 0 ? 0 : (std::uint32_t)ram_ptr;
         if (r.slot0 + n > q.slots) return fail(std::string(fn) + ": ram pointer past the end of '" + q.desc.queue_name + "'");
@@ -400,8 +403,9 @@ DEVICE_STATUS_CODE reserve_write(Queue &q, std::uint32_t n, int timeout_s, int r
 }
 
 // Makes the reserved entries visible, once every earlier reservation has been.  After a failure the slots are given up
-// again if nobody reserved behind them; otherwise they are published as they are, so that the ring stays whole (a failing
-// HIP call leaves the process without a usable device anyway).
+// again if nobody reserved behind them; otherwise they have to be published so that the ring stays whole, but they are
+// marked as never written: a reader of such an entry gets an error instead of stale bytes, and pop_output releases it
+// like any other.
 void publish_write(Queue &q, const Reservation &r, bool ok)
 {
     std::unique_lock<std::mutex> l(q.m);
@@ -409,29 +413,41 @@ void publish_write(Queue &q, const Reservation &r, bool ok)
     if (r.ring) {
         q.cv.wait(l, [&] { return q.ticket_done == r.ticket; });
         q.reserved -= r.n;
-        if (ok || q.ticket_next != r.ticket + 1) {
+        const bool last = q.ticket_next == r.ticket + 1;  // nobody has reserved behind these slots
+        if (ok || !last) {
+            if (!ok)
+                for (std::uint32_t i = 0; i < r.n; ++i) q.poisoned[(r.slot0 + i) % q.slots] = 1;
             q.wr = (q.wr + r.n) % q.slots;
             q.count += r.n;
         }
-        if (!ok && q.ticket_next == r.ticket + 1) q.ticket_next = r.ticket;  // the rollback hands the ticket back too
+        if (!ok && last) q.ticket_next = r.ticket;  // the rollback hands the ticket back too
         else q.ticket_done += 1;
+    } else if (!ok) {
+        for (std::uint32_t i = 0; i < r.n; ++i) q.poisoned[r.slot0 + i] = 1;  // a RAM slot that was only partly rewritten
     }
     q.cv.notify_all();
 }
 
 // Pins n entries for reading: the oldest n of a ring (waits up to timeout_s for them; rd_ptr >= 0 names the first slot
-// instead), or slots rd_ptr.. of a RAM.
-DEVICE_STATUS_CODE begin_read(Queue &q, std::uint32_t n, int timeout_s, int rd_ptr, std::uint32_t &slot0, const char *fn)
+// instead), or slots rd_ptr.. of a RAM.  consume: the caller will pop the entry it reads (end_consume); only one such
+// reader owns the head of a ring at a time, the next one waits for it and then sees the following entry.
+DEVICE_STATUS_CODE begin_read(Queue &q, std::uint32_t n, int timeout_s, int rd_ptr, std::uint32_t &slot0, const char *fn, bool consume = false)
 {
     std::unique_lock<std::mutex> l(q.m);
     if (q.desc.io_type == IO_TYPE::Queue) {
-        if (!wait_until(l, q.cv, timeout_s, [&] { return q.count >= n; }))
-            return fail(std::string(fn) + ": queue '" + q.desc.queue_name + "' is empty", DEVICE_STATUS_CODE::TimeoutError);
+        if (!wait_until(l, q.cv, timeout_s, [&] { return q.count >= n && !(consume && q.consuming); }))
+            return fail(std::string(fn) + ": queue '" + q.desc.queue_name + (q.count >= n ? "' is being consumed" : "' is empty"),
+                        DEVICE_STATUS_CODE::TimeoutError);
         slot0 = rd_ptr >= 0 ? (std::uint32_t)rd_ptr % q.slots : q.rd;
     } else {
         slot0 = rd_ptr < 0 ? 0 : (std::uint32_t)rd_ptr;
         if (slot0 + n > q.slots) return fail(std::string(fn) + ": read pointer past the end of '" + q.desc.queue_name + "'");
     }
+    for (std::uint32_t i = 0; i < n; ++i)
+        if (q.poisoned[(slot0 + i) % q.slots])
+            return fail(std::string(fn) + ": entry " + std::to_string((slot0 + i) % q.slots) + " of '" + q.desc.queue_name +
+                        "' was never written: the push that reserved it failed (pop_output releases it)");
+    if (consume && q.desc.io_type == IO_TYPE::Queue) q.consuming = true;
     q.readers += 1;
     q.in_flight += 1;
     q.max_in_flight = std::max(q.max_in_flight, q.in_flight);
@@ -446,6 +462,25 @@ void end_read(Queue &q)
     q.cv.notify_all();
 }
 
+// End of a consuming read: drops the caller's pin and, with pop, releases the entry it read once no other reader holds
+// entries of the ring (as pop_output would).
+void end_consume(Queue &q, bool pop)
+{
+    std::unique_lock<std::mutex> l(q.m);
+    q.readers -= 1;
+    q.in_flight -= 1;
+    if (q.desc.io_type == IO_TYPE::Queue) {
+        if (pop) {
+            q.cv.wait(l, [&] { return q.readers == 0; });  // readers hold their pin for bounded GPU work only
+            q.poisoned[q.rd] = 0;
+            q.rd = (q.rd + 1) % q.slots;
+            q.count -= 1;
+        }
+        q.consuming = false;
+    }
+    q.cv.notify_all();
+}
+
 // Releases the oldest n entries of a ring (waits up to timeout_s for them and for readers that still hold them).
 DEVICE_STATUS_CODE release_entries(Queue &q, std::uint32_t n, int timeout_s, const char *fn)
 {
@@ -453,6 +488,7 @@ DEVICE_STATUS_CODE release_entries(Queue &q, std::uint32_t n, int timeout_s, con
     if (!wait_until(l, q.cv, timeout_s, [&] { return q.count >= n && q.readers == 0; }))
         return fail(std::string(fn) + ": queue '" + q.desc.queue_name + (q.count >= n ? "' is being read" : "' is empty"),
                     DEVICE_STATUS_CODE::TimeoutError);
+    for (std::uint32_t i = 0; i < n; ++i) q.poisoned[(q.rd + i) % q.slots] = 0;
     q.rd = (q.rd + n) % q.slots;
     q.count -= n;
     q.cv.notify_all();
@@ -565,6 +601,7 @@ tt_dram_io_desc tt_backend::create_queue(const std::string &name, DataFormat for
     if (q->entry_bytes > 0xffffffffull) throw std::runtime_error("create_queue: one entry exceeds 4 GiB");
     d.bufq_entry_size = (std::uint32_t)q->entry_bytes;
     q->slots = num_slots;
+    q->poisoned.assign(num_slots, 0);
     q->pitch = q->entry_bytes * num_slots;
     void *base = nullptr;
     if (ttbfp_alloc(q->pitch * q->buffers, &base) != TTBFP_SUCCESS)
@@ -618,6 +655,19 @@ std::uint32_t tt_backend::queue_max_in_flight(const std::string &name) const
     return q->max_in_flight;
 }
 
+std::uint32_t tt_backend::queue_in_flight(const std::string &name) const
+{
+    std::shared_ptr<Queue> q;
+    {
+        std::lock_guard<std::mutex> l(g_registry_mutex);
+        auto it = g_registry.find(id_ + "/" + name);
+        if (it == g_registry.end()) throw std::runtime_error("queue_in_flight: no queue named '" + name + "'");
+        q = it->second;
+    }
+    std::lock_guard<std::mutex> l(q->m);
+    return q->in_flight;
+}
+
 DEVICE_STATUS_CODE tt_backend::run_matmul(const std::string &in0, const std::string &weight, const std::string &bias,
                                           const std::string &out, bool gelu, int timeout_s, const std::string &approximate)
 {
@@ -656,10 +706,11 @@ DEVICE_STATUS_CODE tt_backend::run_matmul(const std::string &in0, const std::str
     TT_TRY(staging().take((std::uint64_t)M * N * isz, &y.p));
 
     std::uint32_t in_slot = 0;
-    TT_TRY(begin_read(*qa, 1, timeout_s, -1, in_slot, "run_matmul"));
-    struct ReadPin {
+    TT_TRY(begin_read(*qa, 1, timeout_s, -1, in_slot, "run_matmul", true));
+    struct ReadPin {  // the activation entry is this call's until it ends: popped on success, left in place otherwise
         Queue &q;
-        ~ReadPin() { end_read(q); }
+        bool pop = false;
+        ~ReadPin() { end_consume(q, pop); }
     } pin{*qa};
     {
         const std::uint64_t st[4] = {(std::uint64_t)M * K * isz, (std::uint64_t)M * K * isz, (std::uint64_t)K * isz, isz};
@@ -693,12 +744,7 @@ DEVICE_STATUS_CODE tt_backend::run_matmul(const std::string &in0, const std::str
     if (s == DEVICE_STATUS_CODE::Success) s = sync_thread_stream(0);
     publish_write(*qo, r, s == DEVICE_STATUS_CODE::Success);
     TT_TRY(s);
-    if (qa->desc.io_type == IO_TYPE::Queue) {
-        std::lock_guard<std::mutex> l(qa->m);
-        qa->rd = (qa->rd + 1) % qa->slots;
-        qa->count -= 1;
-        qa->cv.notify_all();
-    }
+    pin.pop = true;
     return DEVICE_STATUS_CODE::Success;
 }
 

@@ -154,6 +154,8 @@ class tt_backend {
     DataFormat queue_storage_format(const std::string &name) const;
     // The largest number of push_input / get_output / run_matmul conversions that ever ran on this queue at one time.
     std::uint32_t queue_max_in_flight(const std::string &name) const;
+    // conversions (pushes and reads) of the queue that hold a reservation or a pin right now
+    std::uint32_t queue_in_flight(const std::string &name) const;
     const tt_backend_config &config() const { return config_; }
 
     // out = epilogue(in0 * weight + bias): the matmul op of a netlist program, evaluated with the

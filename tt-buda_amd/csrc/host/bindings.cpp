@@ -284,6 +284,7 @@ void bind_backend(py::module &m)
         .def("get_config", &tt_backend::config)
         .def("queue_storage_format", &tt_backend::queue_storage_format)
         .def("queue_max_in_flight", &tt_backend::queue_max_in_flight)
+        .def("queue_in_flight", &tt_backend::queue_in_flight)
         .def("initialize", &tt_backend::initialize, py::call_guard<py::gil_scoped_release>())
         .def("finish", &tt_backend::finish)
         .def("wait_for_idle", &tt_backend::wait_for_idle, py::call_guard<py::gil_scoped_release>())
