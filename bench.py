@@ -54,6 +54,9 @@ def parse():
     p.add_argument("--no-gemm", action="store_true", help="skip the GEMM / FFN section")
     p.add_argument("--eager-timing", action="store_true", help="time every launch eagerly, no HIP graph (for counter runs)")
     p.add_argument("--gemm-only", action="store_true", help="skip the streaming section's secondary lines (fp32 sources, queue forms)")
+    p.add_argument("--sustained-seconds", type=float, default=2.0,
+                   help="length of the sustained 8192^3 loops whose clock and power are sampled (0: skip them)")
+    p.add_argument("--no-host-push", action="store_true", help="skip the host push / read-back lines (PCIe inclusive)")
     p.add_argument("--power-probe", type=float, default=0.0, metavar="SECONDS",
                    help="instead of the benchmark: run each 8192^3 GEMM form (fused, with workspace, the vendor library's plain bf16 "
                         "GEMM through torch.matmul) back to back for SECONDS while rocm-smi is polled for clock and power; prints one JSON line")
@@ -124,6 +127,59 @@ def power_probe(seconds, torch, capi):
                       "max_clock_mhz": 2400, "forms": out}))
 
 
+def sustained(fn, seconds, flops, torch):
+    """fn() launched back to back for `seconds` while amd-smi is polled: average launch time over the whole run and the
+    median XCD clock and socket power of its second half (the part has then settled into its power limit)."""
+    import re
+    import subprocess
+    import threading
+
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            try:
+                txt = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=20).stdout
+            except Exception:
+                return
+            xcd = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK: (\d+) MHz", txt)]
+            watts = re.search(r"SOCKET_POWER: ([0-9.]+) W", txt)
+            samples.append((time.perf_counter(), sum(xcd) / len(xcd) if xcd else None, float(watts.group(1)) if watts else None))
+            stop.wait(0.1)
+
+    th = threading.Thread(target=poll)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    launches = 0
+    th.start()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            fn()
+        launches += 50
+        torch.cuda.synchronize()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    stop.set()
+    th.join()
+    ms = e0.elapsed_time(e1) / launches
+    late = [(c, w) for t, c, w in samples if t0 + (t1 - t0) / 2 <= t <= t1]  # sampled while the loop ran, second half
+    clocks = sorted(c for c, _ in late if c)
+    watts = sorted(w for _, w in late if w)
+    tf = flops / ms / 1e9
+    clock = clocks[len(clocks) // 2] if clocks else None
+    return {"seconds": round(t1 - t0, 2), "launches": launches, "ms": round(ms, 4), "tflops": round(tf, 1),
+            "frac_of_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "samples": len(late),
+            "clock_mhz": round(clock) if clock else None, "power_w": watts[len(watts) // 2] if watts else None,
+            # what the matrix cores deliver at the clock the part ran at: 256 CUs x 4 SIMDs x 1024 flop per clock
+            "mfma_peak_at_clock_tflops": round(256 * 4 * 1024 * clock * 1e6 / 1e12, 1) if clock else None,
+            "frac_of_peak_at_clock": round(tf / (256 * 4 * 1024 * clock * 1e6 / 1e12), 4) if clock else None}
+
+
 def time_kernel(fn, steps, warmup, torch):
     """(average, minimum) duration of fn() in ms by HIP events on the stream the kernels are launched on.  The average
     comes from one pair of events around `steps` back-to-back launches (an event between launches would put its own
@@ -174,6 +230,62 @@ def time_launches(fn, steps, warmup, torch):
         print("bench.py: graph timing unavailable (%s)" % exc, file=sys.stderr)
         torch.cuda.synchronize()
         return None
+
+
+def host_push_lines(torch):
+    """push_input of a pinned host tensor into a Bfp8_b queue and get_output back, through the host layer, host link
+    included: the figure the reference publishes for its own push path (8.7 GB/s fp32 / fp16, 8.9 GB/s bf16 on chip 0:
+    pybuda/test/galaxy/utils/verify_push_bandwidth.py:10-12) on its own shapes
+    (pybuda/test/galaxy/test_galaxy_inputs.py:119) and on 128 MiB.  GB/s of row-major bytes on the host side.  These
+    lines are PCIe bound and are not part of `value`."""
+    from tt_buda_amd import tensor as T
+    from tt_buda_amd._C import DataFormat as DF
+    from tt_buda_amd._C import backend_api as B
+    from tt_buda_amd.backend import BackendAPI
+
+    OK = B.BackendStatusCode.Success
+    api = BackendAPI(0)
+    lines = {"reference_published_gbs": {"float32": 8.7, "float16": 8.7, "bfloat16": 8.9,
+                                         "source": "pybuda/test/galaxy/utils/verify_push_bandwidth.py:10-12 (other hardware)"}}
+    cases = [("galaxy_shape1_32x1x128x128", (32, 1, 128, 128)), ("galaxy_shape2_256x1x1028x384", (256, 1, 1028, 384)),
+             ("128MiB", None)]
+    try:
+        for tag, shp in cases:
+            for dtype, dname in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+                shape = shp or ((8, 1, 2048, 2048) if dtype == torch.float32 else (8, 1, 2048, 4096))
+                n, rows, cols = shape[0], (shape[2] + 31) // 32 * 32, (shape[3] + 31) // 32 * 32
+                name = "hostpush_%s_%s" % (tag, dname)
+                q = api.create_queue(name, DF.Bfp8_b, (1, rows, cols), num_slots=n, input_count=n)
+                x = torch.rand(*shape, dtype=torch.float32).to(dtype).pin_memory()
+                desc = T.pytorch_tensor_to_tensor_desc(x)
+                nbytes = x.numel() * x.element_size()
+                push_s, get_s = [], []
+                for it in range(8):
+                    t0 = time.perf_counter()
+                    st = B.push_input(q, desc, False, 5, -1)
+                    t1 = time.perf_counter()
+                    assert st == OK, B.last_error()
+                    out = B.PytorchTensorDesc()
+                    if dtype == torch.float32:
+                        out.format = DF.Float32
+                    t2 = time.perf_counter()
+                    st = B.get_output(q, out, False, 5, -1, shape[2] if shape[2] != rows else 0, shape[3] if shape[3] != cols else 0)
+                    t3 = time.perf_counter()
+                    assert st == OK, B.last_error()
+                    assert list(out.shape) == list(shape), (list(out.shape), shape)
+                    assert B.free_tensor(out) == OK and B.pop_output(q, False, 5) == OK
+                    if it >= 2:  # the first rounds fill the block pools
+                        push_s.append(t1 - t0)
+                        get_s.append(t3 - t2)
+                pm, gm = sorted(push_s)[len(push_s) // 2], sorted(get_s)[len(get_s) // 2]
+                lines["%s_%s" % (tag, dname)] = {"shape": list(shape), "bytes": nbytes, "queue_format": "Bfp8_b",
+                                                 "push_input_ms": round(pm * 1e3, 4), "push_input_gbs": round(nbytes / pm / 1e9, 2),
+                                                 "get_output_ms": round(gm * 1e3, 4), "get_output_gbs": round(nbytes / gm / 1e9, 2)}
+    finally:
+        api.shutdown()
+    lines["note"] = ("pinned host tensor -> push_input (H2D copy + tilize/pack into the queue) and get_output (unpack/untilize + D2H copy into "
+                     "pooled pinned memory); wall clock of the call, median of 6 after 2 warm-up rounds; host link included, never part of `value`")
+    return lines
 
 
 def roofline(bound, achieved, peak, unit, traffic=None):
@@ -321,7 +433,9 @@ def main():
             w = torch.randn(1, 1, K, N, generator=gg, device=dev) * 0.02
             return capi.tilize_pack(w, F.Bfp8_b)
 
-        def gemm_case(M, N, K, seed, workspace=False):
+        ROTATE = 20  # distinct packed weights of a decode-like line: 20 x 17.8 MB = 357 MB, more than L2 and the 256 MB last-level cache hold
+
+        def gemm_case(M, N, K, seed, workspace=False, rotate=False):
             wp = pack_weight(K, N, seed)
             gg = torch.Generator(device=dev).manual_seed(seed + 1)
             a = torch.randn(M, K, generator=gg, device=dev).bfloat16()
@@ -337,8 +451,32 @@ def main():
                     timing, eager_ms, ms = "%d launches back to back in one HIP graph, events around the replay" % args.steps, ms, gms
             flops = 2.0 * M * N * K
             min_bytes = 1.0625 * K * N + 2 * M * K + 2 * M * N
+            out = dict(M=M, N=N, K=K)
+            if rotate:
+                # A weight-streaming line timed on ONE weight measures the caches: an XCD's share of 17.8 MB fits its L2 and the
+                # whole weight fits the last-level cache.  Decode streams a different weight per layer, so the line's figure is
+                # taken over ROTATE distinct weights, launch i on weight i mod ROTATE; the one-weight figure stays beside it.
+                out["cache_resident_ms"] = round(ms, 4)
+                out["cache_resident_note"] = "the same launches on one weight, which stays in L2 and the last-level cache between them"
+                wps = [wp] + [pack_weight(K, N, seed + 100 + i) for i in range(ROTATE - 1)]
+                turn = [0]
+
+                def rotating():
+                    capi.gemm_bfp8b(a, wps[turn[0] % ROTATE], N, out=y)
+                    turn[0] += 1
+
+                steps_r = max(args.steps, ROTATE)
+                rms, mn = time_kernel(rotating, steps_r, args.warmup, torch)
+                timing = "events around %d eager launches over %d distinct weights" % (steps_r, ROTATE)
+                if not args.eager_timing:
+                    turn[0] = 0
+                    gms = time_launches(rotating, steps_r, ROTATE, torch)
+                    if gms is not None:
+                        timing, eager_ms, rms = "%d launches over %d distinct weights back to back in one HIP graph, events around the replay" % (steps_r, ROTATE), rms, gms
+                ms = rms
+                del wps
             tf = flops / (ms * 1e-3) / 1e12
-            out = dict(M=M, N=N, K=K, ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2), timing=timing)
+            out.update(ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2), timing=timing)
             if eager_ms is not None:
                 out["eager_ms"] = round(eager_ms, 4)
             key = ("gemm_8192" if M == N == K == 8192 else "gemm_M%d" % M if N == K == 4096 else "") + ("_ws" if workspace else "")
@@ -350,28 +488,45 @@ def main():
                 out["roofline"] = roofline("hbm", min_bytes / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", traffic)
             else:
                 out["roofline"] = roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", traffic)
+            if M == N == K == 8192 and args.sustained_seconds > 0:
+                # the same launch back to back for a couple of seconds with the XCD clock and the socket power sampled
+                # meanwhile: what the part sustains once it sits at its power limit, and the share of the matrix cores'
+                # peak at the clock it actually ran at
+                out["sustained"] = sustained(lambda: capi.gemm_bfp8b(a, wp, N, out=y, workspace=ws), args.sustained_seconds, flops, torch)
+            return out
+
+        def vendor_case(M, N, K, seed):
+            """Yardstick, not this library: the vendor library's plain bf16 GEMM (torch.matmul) on the same shape, nothing to dequantize."""
+            gg = torch.Generator(device=dev).manual_seed(seed)
+            va = torch.randn(M, K, generator=gg, device=dev).bfloat16()
+            vb = (torch.randn(K, N, generator=gg, device=dev) * 0.02).bfloat16()
+            vy = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            vms, vmn = time_kernel(lambda: torch.matmul(va, vb, out=vy), args.steps, args.warmup, torch)
+            timing = "events around each eager launch"
+            if vms < 0.15 and not args.eager_timing:
+                gms = time_launches(lambda: torch.matmul(va, vb, out=vy), args.steps, args.warmup, torch)
+                if gms is not None:
+                    timing, vms = "%d launches back to back in one HIP graph, events around the replay" % args.steps, gms
+            vtf = 2.0 * M * N * K / vms / 1e9
+            out = dict(M=M, N=N, K=K, ms=round(vms, 4), min_ms=round(vmn, 4), tflops=round(vtf, 2), timing=timing,
+                       roofline=roofline("mfma", vtf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+            if M == N == K == 8192 and args.sustained_seconds > 0:
+                out["sustained"] = sustained(lambda: torch.matmul(va, vb, out=vy), args.sustained_seconds, 2.0 * M * N * K, torch)
             return out
 
         gemm["north_star_8192"] = gemm_case(8192, 8192, 8192, 30)
         gemm["north_star_8192_with_workspace"] = gemm_case(8192, 8192, 8192, 30, workspace=True)
-        # reference point, not this library: the vendor library's plain bf16 GEMM on the same shape (no dequantization at all)
-        gg = torch.Generator(device=dev).manual_seed(31)
-        va = torch.randn(8192, 8192, generator=gg, device=dev).bfloat16()
-        vb = (torch.randn(8192, 8192, generator=gg, device=dev) * 0.02).bfloat16()
-        vy = torch.empty(8192, 8192, dtype=torch.bfloat16, device=dev)
-        vms, vmn = time_kernel(lambda: torch.matmul(va, vb, out=vy), args.steps, args.warmup, torch)
-        vtf = 2.0 * 8192 ** 3 / vms / 1e9
-        gemm["reference_vendor_plain_bf16_gemm_8192"] = dict(M=8192, N=8192, K=8192, ms=round(vms, 4), min_ms=round(vmn, 4), tflops=round(vtf, 2),
-                                                             roofline=roofline("mfma", vtf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
-        del va, vb, vy
-        for M in (32, 512, 8192):
+        gemm["reference_vendor_plain_bf16_gemm_8192"] = vendor_case(8192, 8192, 8192, 31)
+        gemm["config4_M32"] = gemm_case(32, 4096, 4096, 3, rotate=True)
+        for M in (512, 8192):
             gemm[f"config4_M{M}"] = gemm_case(M, 4096, 4096, 3)
+        gemm["reference_vendor_plain_bf16_gemm_M512"] = vendor_case(512, 4096, 4096, 32)
         gemm["config4_M8192_with_workspace"] = gemm_case(8192, 4096, 4096, 3, workspace=True)
         # few macro tiles: with a workspace K is split over more workgroups (M = 512 no longer qualifies: its fused form is level)
         gemm["weights4096_M256"] = gemm_case(256, 4096, 4096, 3)
         gemm["weights4096_M256_with_workspace"] = gemm_case(256, 4096, 4096, 3, workspace=True)
         for M in (64, 128):  # between the decode-like and the prefill-like case of config 4
-            gemm[f"weights4096_M{M}"] = gemm_case(M, 4096, 4096, 3)
+            gemm[f"weights4096_M{M}"] = gemm_case(M, 4096, 4096, 3, rotate=True)
 
         gemm["general_kernel_M512_N4128"] = gemm_case(512, 4128, 4096, 3)  # N is no multiple of 64: the bounds-checked general kernel
 
@@ -394,6 +549,18 @@ def main():
         tf = flops / (ms * 1e-3) / 1e12
         gemm["config5_bert_large_ffn"] = dict(ms=round(ms, 4), min_ms=round(mn, 4), tflops=round(tf, 2),
                                               roofline=roofline("mfma", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", MEASURED_TRAFFIC_BYTES["ffn"]))
+        del w1, w2, xa, h, y
+        # the vendor library's plain bf16 GEMM on the FFN's two matmuls (no bias, no GELU, nothing to dequantize)
+        gemm["reference_vendor_plain_bf16_gemm_ffn1"] = vendor_case(3072, 4096, 1024, 53)
+        gemm["reference_vendor_plain_bf16_gemm_ffn2"] = vendor_case(3072, 1024, 4096, 54)
+        vsum = gemm["reference_vendor_plain_bf16_gemm_ffn1"]["ms"] + gemm["reference_vendor_plain_bf16_gemm_ffn2"]["ms"]
+        gemm["reference_vendor_plain_bf16_gemm_ffn_sum"] = dict(ms=round(vsum, 4), tflops=round(flops / vsum / 1e9, 2),
+                                                                note="sum of the two matmul lines above, each timed alone")
+
+    host_push = None
+    if not args.no_host_push:
+        torch.cuda.synchronize()
+        host_push = host_push_lines(torch)
 
     # ---- CPU baseline: the oracle on a bounded sample of the same workload ---------------------------
     cpu_baseline = None
@@ -475,6 +642,7 @@ def main():
         "cpu_baseline": cpu_baseline,
         "kernels": kernels,
         "gemm": gemm,
+        "host_push": host_push,
         "gemm_tflops_8192": gemm.get("north_star_8192", {}).get("tflops"),
         "gemm_frac_of_mfma_peak_8192": gemm.get("north_star_8192", {}).get("roofline", {}).get("frac"),
         "gemm_tflops_8192_with_workspace": gemm.get("north_star_8192_with_workspace", {}).get("tflops"),
