@@ -528,7 +528,12 @@ def main():
         for M in (64, 128):  # between the decode-like and the prefill-like case of config 4
             gemm[f"weights4096_M{M}"] = gemm_case(M, 4096, 4096, 3, rotate=True)
 
-        gemm["general_kernel_M512_N4128"] = gemm_case(512, 4128, 4096, 3)  # N is no multiple of 64: the bounds-checked general kernel
+        # tensors are padded to multiples of 32, not of 64 (pybuda/pybuda/tensor.py:805-877): N an odd number of tiles (all but the
+        # last tile column in the macro-tiled kernel, the last one in one-row-tile workgroups of the weight-streaming kernel),
+        # K an odd number of tile rows (half a slab after the loop), both
+        gemm["ragged_M512_N4128"] = gemm_case(512, 4128, 4096, 3)
+        gemm["ragged_M512_K4128"] = gemm_case(512, 4096, 4128, 3)
+        gemm["ragged_M8192_N4128_K4128"] = gemm_case(8192, 4128, 4128, 3)
 
         # BERT-large FFN: X [3072,1024]; W1 [1024,4096], W2 [4096,1024]
         w1, w2 = pack_weight(1024, 4096, 51), pack_weight(4096, 1024, 52)

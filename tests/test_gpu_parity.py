@@ -371,7 +371,11 @@ def test_gemm_small_against_the_c_oracle():
 @pytest.mark.parametrize("shape", [(32, 96, 160), (32, 1024, 64), (32, 2048, 64), (32, 3072, 32), (64, 3072, 64), (64, 160, 96), (64, 2080, 32), (96, 1504, 192), (128, 256, 384),
                                    (128, 4096, 4096), (160, 96, 224), (224, 128, 256), (608, 192, 384), (416, 160, 96), (256, 512, 256), (384, 192, 640), (512, 1024, 1024),
                                    (768, 128, 16384), (256, 64, 64), (384, 1088, 192), (128 * 17, 128 * 17, 256), (128, 64, 128), (640, 1600, 192), (1024, 2112, 320), (640, 1600, 384), (2048, 1152, 256),
-                                   (1024, 4096, 128), (3072, 4096, 192), (6144, 2048, 64)])
+                                   (1024, 4096, 128), (3072, 4096, 192), (6144, 2048, 64),
+                                   # K an odd number of tile rows (half a slab at the end) in every form of the macro-tiled kernel, and N an odd
+                                   # number of tiles (the last tile column goes to one-row-tile workgroups of the weight-streaming kernel)
+                                   (256, 96, 64), (256, 160, 128), (256, 288, 96), (4224, 96, 576), (3072, 160, 1024), (2176, 96, 2176),
+                                   (3072, 96, 4096), (768, 160, 16384), (416, 224, 224), (512, 4096, 4128), (512, 4128, 4096), (8192, 4128, 4128)])
 def test_gemm_kernel_selection_shapes(shape):
     """One shape per kernel path: one to four tile rows (weight streaming; K that splits unevenly over the wavefronts,
     fewer tile rows of W than wavefronts, slices of one, two, three and four whole tile pairs and of odd counts), ragged (general kernel), 128 x 64

@@ -20,8 +20,10 @@ namespace ttbfp {
 
 hipError_t launch_gemm_bfp8b_general(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
                                      int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
-hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
+hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
                                     int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
+hipError_t launch_gemm_bfp8b_column_rest(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
+                                         int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
 
 static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x 128), 3 (256 x 256 where it fits), all on two stages; 0 / unset: automatic
 {
@@ -29,7 +31,8 @@ static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x
     return force;
 }
 
-static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
+// N columns (from the one w, bias and y point at) of a problem with ldn columns
+static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
                                int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
 {
     if (y_fmt != kFloat32 && y_fmt != kFloat16_b) return hipErrorInvalidValue;
@@ -44,11 +47,11 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
     const auto rounds = [](uint64_t tiles) { return (double)((tiles + TTBFP_CUS - 1) / TTBFP_CUS); };
     if (gemm_fits<TallShape>(M, N, K) && tall_tiles >= TTBFP_BIG_MIN_TILES && (force_tile() == 0 || force_tile() == 5) &&
         (force_tile() == 5 || !big_ok || 0.84 * rounds(tall_tiles) < rounds(big_tiles)))
-        return f32 ? launch_gemm_bfp8b_tall_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                   : launch_gemm_bfp8b_tall_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+        return f32 ? launch_gemm_bfp8b_tall_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_tall_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     if (big_ok && force_tile() != 1 && force_tile() != 2 && force_tile() != 5)
-        return f32 ? launch_gemm_bfp8b_big_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                   : launch_gemm_bfp8b_big_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+        return f32 ? launch_gemm_bfp8b_big_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_big_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     // Fewer tiles than that: which tile and form, by how many workgroups a CU gets.
     //   at most one 128 x 64 workgroup per CU: that tile with two pipelines per workgroup on rings (K a multiple of 128;
     //     else one pipeline on rings) - 512 x 4096 x 4096: 37 us, one pipeline on rings 41, on two stages 49, 128 x 128 54;
@@ -61,47 +64,72 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, const void *x
     static const bool duo = [] { const char *v = getenv("TTBFP_GEMM_PIPELINES"); return !v || atoi(v) != 1; }();
     const uint64_t small_tiles = (uint64_t)(M / 128) * (N / 128), slim_tiles = (uint64_t)(M / 128) * (N / 64);
     if (force == 0 && gemm_fits<SlimShape>(M, N, K) && slim_tiles <= TTBFP_CUS) {
-        if (duo && K % 128 == 0)
-            return f32 ? launch_gemm_bfp8b_duo_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                       : launch_gemm_bfp8b_duo_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
-        return f32 ? launch_gemm_bfp8b_ring_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                   : launch_gemm_bfp8b_ring_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+        if (duo && (K / 64) % 2 == 0)
+            return f32 ? launch_gemm_bfp8b_duo_slim_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                       : launch_gemm_bfp8b_duo_slim_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
+        return f32 ? launch_gemm_bfp8b_ring_slim_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_ring_slim_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     }
-    if (force == 0 && duo && gemm_fits<SmallShape>(M, N, K) && small_tiles <= TTBFP_CUS && K % 128 == 0)
-        return f32 ? launch_gemm_bfp8b_duo_small_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                   : launch_gemm_bfp8b_duo_small_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+    if (force == 0 && duo && gemm_fits<SmallShape>(M, N, K) && small_tiles <= TTBFP_CUS && (K / 64) % 2 == 0)
+        return f32 ? launch_gemm_bfp8b_duo_small_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_duo_small_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     if (gemm_fits<SlimShape>(M, N, K) && (force == 1 || (force == 0 && small_tiles < TTBFP_SLIM_BELOW_TILES)))
-        return f32 ? launch_gemm_bfp8b_slim_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                   : launch_gemm_bfp8b_slim_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+        return f32 ? launch_gemm_bfp8b_slim_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_slim_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     if (gemm_fits<SmallShape>(M, N, K))
-        return f32 ? launch_gemm_bfp8b_small_f32(M, N, K, x, w, bias, epilogue, y, stream)
-                   : launch_gemm_bfp8b_small_bf16(M, N, K, x, w, bias, epilogue, y, stream);
+        return f32 ? launch_gemm_bfp8b_small_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_small_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     return hipErrorNotSupported;  // the caller falls back to the general kernel
+}
+
+// M rows of N columns out of ldn: the macro-tiled kernel where the shape suits a tile, with the last M mod 128 rows
+// (the rows are independent) given to the weight-streaming kernel; hipErrorNotSupported if no tile suits.
+static hipError_t launch_rows_tiled(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
+                                    int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
+{
+    const size_t y_item = y_fmt == kFloat32 ? 4 : 2;
+    hipError_t e = launch_tiled(M, N, K, ldn, x, w, bias, epilogue, y, y_fmt, stream);
+    if (e != hipErrorNotSupported) return e;
+    // M = 128 q + r with 0 < r < 128: the first 128 q rows go to the macro-tiled kernel and the last r (a multiple of 32)
+    // to the weight-streaming one, provided N and K suit the tiles
+    const uint32_t rest = M % 128, body = M - rest;
+    if (body != 0 && rest % 32 == 0 && gemm_fits<SlimShape>(body, N, K)) {
+        e = launch_tiled(body, N, K, ldn, x, w, bias, epilogue, y, y_fmt, stream);
+        if (e != hipSuccess) return e;
+        return launch_gemm_bfp8b_skinny(rest, N, K, ldn, (const uint8_t *)x + (size_t)body * K * 2, w, bias, epilogue,
+                                        (uint8_t *)y + (size_t)body * ldn * y_item, y_fmt, stream);
+    }
+    return hipErrorNotSupported;
 }
 
 hipError_t launch_gemm_bfp8b(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
                              int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
 {
     if (M == 0 || N == 0) return hipSuccess;
-    hipError_t e = launch_gemm_bfp8b_skinny(M, N, K, x, w, bias, epilogue, y, y_fmt, stream);  // M <= 128: weight streaming
+    hipError_t e = launch_gemm_bfp8b_skinny(M, N, K, N, x, w, bias, epilogue, y, y_fmt, stream);  // M <= 128: weight streaming
     if (e != hipErrorNotSupported) return e;
     const size_t y_item = y_fmt == kFloat32 ? 4 : 2;
     if (M < 256 && M % 32 == 0) {  // five to seven tile rows: two passes of the weight-streaming kernel beat one 128-row macro tile
-        e = launch_gemm_bfp8b_skinny(128, N, K, x, w, bias, epilogue, y, y_fmt, stream);
+        e = launch_gemm_bfp8b_skinny(128, N, K, N, x, w, bias, epilogue, y, y_fmt, stream);
         if (e != hipSuccess) return e;
-        return launch_gemm_bfp8b_skinny(M - 128, N, K, (const uint8_t *)x + (size_t)128 * K * 2, w, bias, epilogue,
+        return launch_gemm_bfp8b_skinny(M - 128, N, K, N, (const uint8_t *)x + (size_t)128 * K * 2, w, bias, epilogue,
                                         (uint8_t *)y + (size_t)128 * N * y_item, y_fmt, stream);
     }
-    e = launch_tiled(M, N, K, x, w, bias, epilogue, y, y_fmt, stream);
+    e = launch_rows_tiled(M, N, K, N, x, w, bias, epilogue, y, y_fmt, stream);
     if (e != hipErrorNotSupported) return e;
-    // M = 128 q + r with 0 < r < 128: the rows are independent, so the first 128 q go to the macro-tiled kernel and the
-    // last r (a multiple of 32) to the weight-streaming one, provided N and K suit the tiles
-    const uint32_t rest = M % 128, body = M - rest;
-    if (body != 0 && rest % 32 == 0 && gemm_fits<SmallShape>(body, N, K)) {
-        e = launch_tiled(body, N, K, x, w, bias, epilogue, y, y_fmt, stream);
-        if (e != hipSuccess) return e;
-        return launch_gemm_bfp8b_skinny(rest, N, K, (const uint8_t *)x + (size_t)body * K * 2, w, bias, epilogue,
-                                        (uint8_t *)y + (size_t)body * N * y_item, y_fmt, stream);
+    // N is an odd number of tiles (tensors are padded to multiples of 32, not of 64: pybuda/pybuda/tensor.py:805-877): the
+    // columns but the last 32 go to the macro-tiled kernel, the last tile column to one-row-tile workgroups of the
+    // weight-streaming kernel.  The bias may be fp32 or bf16: the pointer moves by its element size.
+    if (N % 64 == 32 && N > 32 && M % 32 == 0) {
+        const uint32_t body = N - 32;
+        e = launch_rows_tiled(M, body, K, N, x, w, bias, epilogue, y, y_fmt, stream);
+        if (e == hipSuccess) {
+            const size_t bias_item = (epilogue & kEpilogueBiasF32) ? 4 : 2;
+            return launch_gemm_bfp8b_column_rest(M, 32, K, N, x, (const uint8_t *)w + (size_t)(body / kTile) * tile_bytes(kBfp8_b),
+                                                 bias ? (const uint8_t *)bias + (size_t)body * bias_item : nullptr, epilogue,
+                                                 (uint8_t *)y + (size_t)body * y_item, y_fmt, stream);
+        }
+        if (e != hipErrorNotSupported) return e;
     }
     return launch_gemm_bfp8b_general(M, N, K, x, w, bias, epilogue, y, y_fmt, stream);
 }

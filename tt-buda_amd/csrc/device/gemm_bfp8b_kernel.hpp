@@ -29,7 +29,11 @@
 //      direct load fills 8 whole rows, and 16 consecutive rows of one k chunk cover all 64 banks;
 //   B: [k/8][n'][8 k] with n' = n ^ (((n >> 3) ^ (n >> 6)) & 7), which also spreads the vectors a
 //      thread stores (consecutive n) over distinct banks.
-// This kernel has no bounds tests: M % BM == 0, N % BN == 0, K % 64 == 0.  Other shapes take
+// This kernel has no bounds tests: M % BM == 0, N % BN == 0, K % 32 == 0 and K >= 64.  N is the number of columns this
+// launch computes, ldn the number of columns of the whole problem (the pitch of Y's rows and of W's tile rows): a
+// problem whose N does not suit the tiles is cut into column ranges by the host, which offsets the W, Y and bias
+// pointers to the range's first column.  A K that is an odd number of tile rows ends in half a slab, which is multiplied
+// in a short phase of its own after the loop (no overlap: it is one tile row of W and 32 k of X).  Other shapes take
 // gemm_bfp8b_general.hip.
 #pragma once
 
@@ -297,7 +301,7 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi)
 // (both run the same number of iterations) and at the end, where the halves are added through LDS and each pipeline
 // finishes half of the tile's 32 x 32 blocks.  A SIMD then has two wavefronts to issue from.
 template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL = false, bool SPLITK = false, int RING = 0, int GROUPS = 1>
-__global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, uint32_t N, uint32_t K, int epilogue,
+__global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, int epilogue,
                                                            const uint16_t *__restrict__ X,
                                                            const uint8_t *__restrict__ Wp,
                                                            const uint16_t *__restrict__ bias, OutT *__restrict__ Y)
@@ -340,7 +344,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         }
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-    const uint32_t tiles_n = N / kTile;
+    const uint32_t tiles_n = ldn / kTile;  // tiles in a tile row of W
     static_assert(!(SPLITK && PANEL) && (!SPLITK || sizeof(OutT) == 4), "k split: packed W, fp32 partial sums");
     static_assert(RING == 0 || (RING >= 3 && !PANEL && !SPLITK && S::NW == 4), "rings: three or more stages, packed W, four wavefronts");
     const uint32_t split = SPLITK ? blockIdx.y : group;
@@ -782,6 +786,41 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         k_step(integral_constant<int, (4 - AHEAD + decltype(jc)::value) % NBUF>{}, [&](auto) {});
     });
 
+    // ---- half a slab at the end of K (K an odd number of tile rows): k rows K - 32 .. K - 1 ------------------------------
+    // Stage 0 of the first pipeline takes the 32 k of X (the chunks of its upper half are filled with copies and never
+    // read) and the one tile row of W that is left; two k steps multiply them.  Nothing here overlaps: it runs once.
+    if constexpr (!PANEL && !SPLITK) {
+        if (K % BK) {  // uniform
+            __syncthreads();  // every wavefront has read its last operands out of the stages
+            if (group == 0) {
+                const uint32_t tail_slab = K / BK;
+                const uint64_t x_rows = uniform64((uint64_t)(uintptr_t)X + (uint64_t)(m0 + wave * XI * 8) * K * 2 + (uint64_t)tail_slab * (BK * 2));
+                static_for<XI>([&](auto ic) {
+                    constexpr int I = decltype(ic)::value;
+                    const uint32_t chunk = (lane & 7) ^ (lane >> 3) ^ ((wave * XI + I) & 7u);  // the logical chunk this lane's piece stands for
+                    const uint32_t off = (I * 8 + (lane >> 3)) * K * 2 + (chunk & 3u) * 16 - (I % 4) * 1024;  // chunks 4 .. 7 lie past the row: chunk - 4 again
+                    direct_load_16<(I % 4) * 1024>(x_rows, off, lds_base + (wave * XI + I / 4 * 4) * 8 * A_ROW);
+                });
+                uint8_t *const b_stage = RING > 0 ? lds + A_RING - A_BYTES : lds;
+                if ((w_kc >> 2) == 0) {  // the threads whose patch lies in the slab's first tile row; the second does not exist
+                    const uint32_t w_tail_slab = tail_slab - split * nslabs;  // w_src starts at this pipeline's first slab
+                    static_for<WU>([&](auto uc) { fetch_w(w_tail_slab, P0, uc); });
+                    stage_exponents(P0);
+                    static_for<NU>([&](auto kc) { dequant_step(b_stage, P0, kc); });
+                }
+                wait_direct_loads();
+            }
+            __syncthreads();
+            if (group == 0) {
+                uint8_t *const b_stage = RING > 0 ? lds + A_RING - A_BYTES : lds;
+                static_for<2>([&](auto kc) {
+                    static_for<MB + NB>([&](auto uc) { read_one2(lds, b_stage, uc, kc, kc); });
+                });
+                static_for<2>([&](auto kc) { k_step(kc, [&](auto) {}); });
+            }
+        }
+    }
+
     // D layout of the 32x32 MFMA: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
     accumulator_settle<ALL_AGPRS>();
     // two pipelines: block BLK is finished by pipeline BLK % 2, which gets the other one's partial sums through LDS
@@ -825,11 +864,11 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
                 *(uint16_t *)(ip + rr1 * PITCH) = (uint16_t)(pair >> 16);
             });
         } else {
-            OutT *yp = Y + (uint64_t)(m0 + row_in_tile) * N + n0 + col_in_tile;
+            OutT *yp = Y + (uint64_t)(m0 + row_in_tile) * ldn + n0 + col_in_tile;
             static_for<16>([&](auto rc) {
                 constexpr int r = decltype(rc)::value;
                 constexpr uint32_t rr = (r >> 2) * 8 + (r & 3);
-                yp[(uint64_t)rr * N] = finished(bc, rc, bv);
+                yp[(uint64_t)rr * ldn] = finished(bc, rc, bv);
             });
         }
     });
@@ -840,8 +879,8 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         static_assert(BM % RPP == 0, "whole passes");
         const uint32_t row = threadIdx.x / LPR, piece = threadIdx.x % LPR;
         const uint8_t *from = image + row * PITCH + piece * 16;
-        uint8_t *to = (uint8_t *)Y + ((uint64_t)(m0 + row) * N + n0) * 2 + piece * 16;
-        const uint64_t step = (uint64_t)RPP * N * 2;
+        uint8_t *to = (uint8_t *)Y + ((uint64_t)(m0 + row) * ldn + n0) * 2 + piece * 16;
+        const uint64_t step = (uint64_t)RPP * ldn * 2;
         static_for<BM / RPP>([&](auto pc) {
             constexpr int PASS = decltype(pc)::value;
             *(uint4 *)(to + PASS * step) = *(const uint4 *)(from + PASS * RPP * PITCH);
@@ -850,7 +889,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
 }
 
 template <typename S, typename OutT, bool XCD_BLOCKS, bool PANEL, int GROUPS = 1>
-hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
+hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, int epilogue,
                        void *y, hipStream_t stream)
 {
     constexpr uint32_t smem = workgroup_lds_bytes<S, OutT, PANEL, 0, GROUPS>();
@@ -861,13 +900,13 @@ hipError_t launch_tile(uint32_t M, uint32_t N, uint32_t K, const void *x, const 
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
     const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);  // the walk in eighths: see the kernel
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT * GROUPS), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT * GROUPS), smem, stream, M, N, K, ldn, epilogue, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
     return hipGetLastError();
 }
 
 template <typename S, typename OutT, bool XCD_BLOCKS, int LA, int GROUPS = 1>
-hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
+hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, int epilogue,
                             void *y, hipStream_t stream)
 {
     constexpr uint32_t smem = workgroup_lds_bytes<S, OutT, false, LA, GROUPS>();
@@ -878,19 +917,19 @@ hipError_t launch_tile_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, c
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
     if (tiles > 0x7ffffff0ull) return hipErrorInvalidValue;
     const uint32_t grid = XCD_BLOCKS ? (uint32_t)tiles : (uint32_t)((tiles + 7) / 8 * 8);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT * GROUPS), smem, stream, M, N, K, epilogue, (const uint16_t *)x,
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(S::NT * GROUPS), smem, stream, M, N, K, ldn, epilogue, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, (OutT *)y);
     return hipGetLastError();
 }
 
 template <typename S, typename OutT, int LA, int GROUPS = 1>
-hipError_t launch_shape_ring(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
+hipError_t launch_shape_ring(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, int epilogue,
                              void *y, hipStream_t stream)
 {
     const uint32_t gm = M / S::BM, gn = N / S::BN;
     if (gm % 4 == 0 && gn % 8 == 0 && ((gm / 4) * (gn / 8)) % 8 == 0)
-        return launch_tile_ring<S, OutT, true, LA, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
-    return launch_tile_ring<S, OutT, false, LA, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
+        return launch_tile_ring<S, OutT, true, LA, GROUPS>(M, N, K, ldn, x, w, bias, epilogue, y, stream);
+    return launch_tile_ring<S, OutT, false, LA, GROUPS>(M, N, K, ldn, x, w, bias, epilogue, y, stream);
 }
 
 // k split: `splits` workgroups per tile, fp32 partial planes [splits][M][N] at `partials`
@@ -902,8 +941,8 @@ hipError_t launch_tile_splitk(uint32_t M, uint32_t N, uint32_t K, uint32_t split
     auto kernel = gemm_bfp8b_kernel<S, float, false, false, true>;
     if (hipError_t e = allow_dynamic_lds(kernel, smem); e != hipSuccess) return e;
     const uint64_t tiles = (uint64_t)(N / S::BN) * (M / S::BM);
-    if (tiles > 0x7fffffffull || splits == 0 || splits > 65535 || (K / BK) % splits) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles, splits), dim3(S::NT), smem, stream, M, N, K, 0, (const uint16_t *)x,
+    if (tiles > 0x7fffffffull || splits == 0 || splits > 65535 || K % BK || (K / BK) % splits) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles, splits), dim3(S::NT), smem, stream, M, N, K, N, 0, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)nullptr, partials);
     return hipGetLastError();
 }
@@ -912,18 +951,19 @@ hipError_t launch_tile_splitk(uint32_t M, uint32_t N, uint32_t K, uint32_t split
 template <typename S>
 bool fits(uint32_t M, uint32_t N, uint32_t K)
 {
-    return M % S::BM == 0 && N % S::BN == 0 && K % BK == 0 && K <= (1u << 24);  // 32-bit X offsets inside a wave's rows
+    return M % S::BM == 0 && N % S::BN == 0 && K % kTile == 0 && K >= BK && K <= (1u << 24);  // 32-bit X offsets inside a wave's rows
 }
 
 template <typename S, typename OutT, bool PANEL = false, int GROUPS = 1>
-hipError_t launch_shape(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue,
+hipError_t launch_shape(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, int epilogue,
                         void *y, hipStream_t stream)
 {
+    if (PANEL && (K % BK || ldn != N)) return hipErrorInvalidValue;  // the panel is made for whole slabs of the whole weight
     // 4 x 8 blocks of tiles per XCD need a whole number of rounds of 8 blocks
     const uint32_t gm = M / S::BM, gn = N / S::BN;
     if (gm % 4 == 0 && gn % 8 == 0 && ((gm / 4) * (gn / 8)) % 8 == 0)
-        return launch_tile<S, OutT, true, PANEL, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
-    return launch_tile<S, OutT, false, PANEL, GROUPS>(M, N, K, x, w, bias, epilogue, y, stream);
+        return launch_tile<S, OutT, true, PANEL, GROUPS>(M, N, K, ldn, x, w, bias, epilogue, y, stream);
+    return launch_tile<S, OutT, false, PANEL, GROUPS>(M, N, K, ldn, x, w, bias, epilogue, y, stream);
 }
 
 }  // namespace
@@ -952,7 +992,7 @@ inline bool gemm_fits(uint32_t M, uint32_t N, uint32_t K)
 
 // defined by the per-shape translation units; y_is_fp32 selects the Float32 (else Float16_b) output
 #define TTBFP_DECLARE_GEMM(NAME)                                                                                        \
-    hipError_t launch_gemm_bfp8b_##NAME(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, \
+    hipError_t launch_gemm_bfp8b_##NAME(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, \
                                         int epilogue, void *y, hipStream_t stream)
 TTBFP_DECLARE_GEMM(big_f32);
 TTBFP_DECLARE_GEMM(big_bf16);
@@ -973,14 +1013,14 @@ TTBFP_DECLARE_GEMM(panel_bf16);
 TTBFP_DECLARE_GEMM(panel_small_f32);  // SmallShape on a panel made for 128-wide tiles
 TTBFP_DECLARE_GEMM(panel_small_bf16);
 #define TTBFP_DEFINE_PANEL_GEMM(NAME, SHAPE, OUT_T)                                                                    \
-    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, true>(M, N, K, x, w, bias, epilogue, y, stream); }
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, true>(M, N, K, ldn, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_RING_GEMM(NAME, SHAPE, OUT_T, LA)                                                                 \
-    TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA>(M, N, K, x, w, bias, epilogue, y, stream); }
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA>(M, N, K, ldn, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_DUO_GEMM(NAME, SHAPE, OUT_T, LA)                                                                  \
-    TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA, 2>(M, N, K, x, w, bias, epilogue, y, stream); }
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape_ring<SHAPE, OUT_T, LA, 2>(M, N, K, ldn, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_DUO_STAGED_GEMM(NAME, SHAPE, OUT_T)                                                               \
-    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, false, 2>(M, N, K, x, w, bias, epilogue, y, stream); }
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T, false, 2>(M, N, K, ldn, x, w, bias, epilogue, y, stream); }
 #define TTBFP_DEFINE_GEMM(NAME, SHAPE, OUT_T)                                                                          \
-    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T>(M, N, K, x, w, bias, epilogue, y, stream); }
+    TTBFP_DECLARE_GEMM(NAME) { return launch_shape<SHAPE, OUT_T>(M, N, K, ldn, x, w, bias, epilogue, y, stream); }
 
 }  // namespace ttbfp

@@ -86,6 +86,7 @@ __global__ __launch_bounds__(64 * kPanelWaves) void dequant_panel_kernel(uint32_
 // The conversion costs about 3 bytes of traffic per weight; it pays once enough rows share it.
 static uint32_t panel_tile(uint32_t M, uint32_t N, uint32_t K)
 {
+    if (K % 64) return 0;  // the panel is cut into whole slabs
     const uint64_t big_tiles = (uint64_t)(M / 256) * (N / 256);
     if (gemm_fits<BigShape>(M, N, K) && big_tiles >= TTBFP_PANEL_BIG_MIN_TILES) return M >= TTBFP_PANEL_BIG_MIN_M ? 256 : 0;
     if (gemm_fits<SmallShape>(M, N, K)) return M >= TTBFP_PANEL_SMALL_MIN_M ? 128 : 0;
@@ -105,10 +106,10 @@ hipError_t launch_gemm_bfp8b_panel(uint32_t M, uint32_t N, uint32_t K, const voi
                        (const uint8_t *)w, (uint8_t *)workspace, tile);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (tile == 256)
-        return y_fmt == kFloat32 ? launch_gemm_bfp8b_panel_f32(M, N, K, x, workspace, bias, epilogue, y, stream)
-                                 : launch_gemm_bfp8b_panel_bf16(M, N, K, x, workspace, bias, epilogue, y, stream);
-    return y_fmt == kFloat32 ? launch_gemm_bfp8b_panel_small_f32(M, N, K, x, workspace, bias, epilogue, y, stream)
-                             : launch_gemm_bfp8b_panel_small_bf16(M, N, K, x, workspace, bias, epilogue, y, stream);
+        return y_fmt == kFloat32 ? launch_gemm_bfp8b_panel_f32(M, N, K, N, x, workspace, bias, epilogue, y, stream)
+                                 : launch_gemm_bfp8b_panel_bf16(M, N, K, N, x, workspace, bias, epilogue, y, stream);
+    return y_fmt == kFloat32 ? launch_gemm_bfp8b_panel_small_f32(M, N, K, N, x, workspace, bias, epilogue, y, stream)
+                             : launch_gemm_bfp8b_panel_small_bf16(M, N, K, N, x, workspace, bias, epilogue, y, stream);
 }
 
 }  // namespace ttbfp

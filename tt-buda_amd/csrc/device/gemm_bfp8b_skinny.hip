@@ -52,7 +52,7 @@ typedef __attribute__((address_space(3))) v2i *lds_v2i;
 
 
 template <int RT, int EPILOGUE, typename OutT>
-__global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_kernel(uint32_t N, uint32_t K,
+__global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_kernel(uint32_t ldn, uint32_t K,
                                                                         const uint16_t *__restrict__ X,
                                                                         const uint8_t *__restrict__ Wp,
                                                                         const uint16_t *__restrict__ bias, int bias_f32,
@@ -63,7 +63,11 @@ __global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_ker
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // kWaves regions of kRegion bytes
 
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t tiles_n = N / kTile, tiles_k = K / kTile;
+    // ldn: columns of the whole problem (the pitch of Y's rows and of W's tile rows).  The launch computes the columns from
+    // the one W, Y and bias point at: gridDim.x / 2 tile columns, and gridDim.y groups of RT row tiles.
+    const uint32_t tiles_n = ldn / kTile, tiles_k = K / kTile;
+    X += (uint64_t)blockIdx.y * (RT * 32) * K;
+    Y += (uint64_t)blockIdx.y * (RT * 32) * ldn;
     // Tile column, and its left (0) or right (1) faces.  Workgroups go to the XCDs in turn (id mod 8), and the two halves
     // of a tile column share the lines that straddle two faces, so they are ids b and b + 8: same XCD, same L2.
     uint32_t nt = blockIdx.x >> 1, half = blockIdx.x & 1;
@@ -200,53 +204,77 @@ __global__ __launch_bounds__(64 * Skinny<RT>::kWaves) void gemm_bfp8b_skinny_ker
         if (bias) v += load_bias(bias, col, bias_f32);
         v = apply_epilogue(EPILOGUE, v);
         if constexpr (sizeof(OutT) == 4)
-            Y[(uint64_t)row * N + col] = v;
+            Y[(uint64_t)row * ldn + col] = v;
         else
-            Y[(uint64_t)row * N + col] = f32_to_bf16_rne(__float_as_uint(v));
+            Y[(uint64_t)row * ldn + col] = f32_to_bf16_rne(__float_as_uint(v));
     }
 }
 
 template <int RT, int EPILOGUE, typename OutT>
-hipError_t launch(uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int bias_f32, void *y, hipStream_t stream)
+hipError_t launch(uint32_t groups, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, int bias_f32, void *y,
+                  hipStream_t stream)
 {
     constexpr uint32_t smem = Skinny<RT>::kWaves * Skinny<RT>::kRegion;
     auto kernel = gemm_bfp8b_skinny_kernel<RT, EPILOGUE, OutT>;
+    if (groups == 0 || groups > 65535u) return hipErrorInvalidValue;
     if (hipError_t e = allow_dynamic_lds(kernel, smem); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3(N / kTile * 2), dim3(64 * Skinny<RT>::kWaves), smem, stream, N, K, (const uint16_t *)x,
+    hipLaunchKernelGGL(kernel, dim3(N / kTile * 2, groups), dim3(64 * Skinny<RT>::kWaves), smem, stream, ldn, K, (const uint16_t *)x,
                        (const uint8_t *)w, (const uint16_t *)bias, bias_f32, (OutT *)y);
     return hipGetLastError();
 }
 
+// groups x RT row tiles of X, N columns from the one the pointers are at
 template <int RT>
-hipError_t launch_rows(uint32_t N, uint32_t K, const void *x, const void *w, const void *bias, int epilogue, void *y, uint8_t y_fmt,
-                       hipStream_t stream)
+hipError_t launch_rows(uint32_t groups, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias, int epilogue, void *y,
+                       uint8_t y_fmt, hipStream_t stream)
 {
     const int bias_f32 = epilogue & kEpilogueBiasF32;
     epilogue &= kEpilogueMask;
     if (y_fmt == kFloat32)
-        return epilogue == 2   ? launch<RT, 2, float>(N, K, x, w, bias, bias_f32, y, stream)
-               : epilogue == 1 ? launch<RT, 1, float>(N, K, x, w, bias, bias_f32, y, stream)
-                               : launch<RT, 0, float>(N, K, x, w, bias, bias_f32, y, stream);
+        return epilogue == 2   ? launch<RT, 2, float>(groups, N, K, ldn, x, w, bias, bias_f32, y, stream)
+               : epilogue == 1 ? launch<RT, 1, float>(groups, N, K, ldn, x, w, bias, bias_f32, y, stream)
+                               : launch<RT, 0, float>(groups, N, K, ldn, x, w, bias, bias_f32, y, stream);
     if (y_fmt == kFloat16_b)
-        return epilogue == 2   ? launch<RT, 2, uint16_t>(N, K, x, w, bias, bias_f32, y, stream)
-               : epilogue == 1 ? launch<RT, 1, uint16_t>(N, K, x, w, bias, bias_f32, y, stream)
-                               : launch<RT, 0, uint16_t>(N, K, x, w, bias, bias_f32, y, stream);
+        return epilogue == 2   ? launch<RT, 2, uint16_t>(groups, N, K, ldn, x, w, bias, bias_f32, y, stream)
+               : epilogue == 1 ? launch<RT, 1, uint16_t>(groups, N, K, ldn, x, w, bias, bias_f32, y, stream)
+                               : launch<RT, 0, uint16_t>(groups, N, K, ldn, x, w, bias, bias_f32, y, stream);
     return hipErrorInvalidValue;
 }
 
 }  // namespace
 
-// M = 32, 64, 96 or 128; returns hipErrorNotSupported otherwise so that the caller picks another kernel.
-hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, const void *x, const void *w, const void *bias,
+// M = 32, 64, 96 or 128 rows and N columns of a problem with ldn columns (w, bias and y point at the first of the N);
+// returns hipErrorNotSupported for another M so that the caller picks another kernel.
+hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
                                     int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
 {
     switch (M) {
-        case 32: return launch_rows<1>(N, K, x, w, bias, epilogue, y, y_fmt, stream);
-        case 64: return launch_rows<2>(N, K, x, w, bias, epilogue, y, y_fmt, stream);
-        case 96: return launch_rows<3>(N, K, x, w, bias, epilogue, y, y_fmt, stream);
-        case 128: return launch_rows<4>(N, K, x, w, bias, epilogue, y, y_fmt, stream);
+        case 32: return launch_rows<1>(1, N, K, ldn, x, w, bias, epilogue, y, y_fmt, stream);
+        case 64: return launch_rows<2>(1, N, K, ldn, x, w, bias, epilogue, y, y_fmt, stream);
+        case 96: return launch_rows<3>(1, N, K, ldn, x, w, bias, epilogue, y, y_fmt, stream);
+        case 128: return launch_rows<4>(1, N, K, ldn, x, w, bias, epilogue, y, y_fmt, stream);
         default: return hipErrorNotSupported;
     }
+}
+
+// Any number of rows (a multiple of 32) of a few columns: the column range a macro-tiled launch leaves over.  One row
+// tile per workgroup, M / 32 groups of them: each streams its 16 columns of W over all of K, so the launch takes about
+// as long as one decode-like call however many rows there are, as long as the workgroups fit the CUs at once.
+hipError_t launch_gemm_bfp8b_column_rest(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
+                                         int epilogue, void *y, uint8_t y_fmt, hipStream_t stream)
+{
+    if (M == 0 || N == 0) return hipSuccess;
+    if (M % kTile || N % kTile) return hipErrorInvalidValue;
+    const uint32_t row_tiles = M / kTile;
+    const size_t y_item = y_fmt == kFloat32 ? 4 : 2;
+    for (uint32_t first = 0; first < row_tiles; first += 65535u) {  // the grid's y dimension holds 65535 groups
+        const uint32_t groups = row_tiles - first < 65535u ? row_tiles - first : 65535u;
+        if (hipError_t e = launch_rows<1>(groups, N, K, ldn, (const uint8_t *)x + (size_t)first * kTile * K * 2, w, bias, epilogue,
+                                          (uint8_t *)y + (size_t)first * kTile * ldn * y_item, y_fmt, stream);
+            e != hipSuccess)
+            return e;
+    }
+    return hipSuccess;
 }
 
 }  // namespace ttbfp

@@ -83,7 +83,7 @@ hipError_t launch_reduce(uint32_t splits, uint64_t quads, uint32_t N, const floa
 // four runs 18.1 / 21.2 (not taken).  The cut with the shortest prediction wins if it saves 3 us or more.
 static uint32_t splitk_factor(uint32_t M, uint32_t N, uint32_t K)
 {
-    if (!gemm_fits<SmallShape>(M, N, K) || M < 256) return 0;  // up to 255 rows go to the weight-streaming kernel
+    if (!gemm_fits<SmallShape>(M, N, K) || K % 64 || M < 256) return 0;  // up to 255 rows go to the weight-streaming kernel
     const uint64_t tiles = (uint64_t)(M / 128) * (N / 128);
     if (tiles > 256) return 0;
     const uint32_t slabs = K / BK;
