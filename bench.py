@@ -423,7 +423,26 @@ def main():
         kernels["tilize_pack_fp32_to_bfp8b_padded_8190x8168"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
         ms, _ = time_kernel(lambda: capi.unpack_untilize_narrow(pk, F.Bfp8_b, ragged.shape, out=ragged), args.steps, args.warmup, torch)
         kernels["unpack_untilize_bfp8b_to_fp32_narrowed_8190x8168"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
-        del wide, strided, ragged, pk
+        del strided, ragged, pk
+        # a sliced view with unit element stride whose first element is one element off a 16-byte boundary
+        # (pybuda/pybuda/tensor.py:707-717): the row kernels with 16-byte accesses that start anywhere
+        view = wide[:, :, :, 1:8161]
+        pk = torch.empty(capi.packed_size(F.Bfp8_b, view.shape), dtype=torch.uint8, device=dev)
+        b = view.numel() * 4 + pk.numel()
+        ms, _ = time_kernel(lambda: capi.tilize_pack(view, F.Bfp8_b, out=pk), args.steps, args.warmup, torch)
+        kernels["tilize_pack_fp32_to_bfp8b_view_off_by_one_element_8192x8160"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        ms, _ = time_kernel(lambda: capi.unpack_untilize(pk, F.Bfp8_b, view.shape, out=view), args.steps, args.warmup, torch)
+        kernels["unpack_untilize_bfp8b_to_fp32_view_off_by_one_element_8192x8160"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        del wide, view, pk
+        xv = x[:, :, :, 1:8161]  # the same on the bf16 workload tensor, 1 GiB
+        pkv = torch.empty(capi.packed_size(F.Bfp8_b, xv.shape), dtype=torch.uint8, device=dev)
+        b = xv.numel() * 2 + pkv.numel()
+        ms, _ = time_kernel(lambda: capi.tilize_pack(xv, F.Bfp8_b, out=pkv), args.steps, args.warmup, torch)
+        kernels["tilize_pack_bf16_to_bfp8b_view_off_by_one_element_8x8192x8160"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        backv = back[:, :, :, 1:8161]
+        ms, _ = time_kernel(lambda: capi.unpack_untilize(pkv, F.Bfp8_b, xv.shape, out=backv), args.steps, args.warmup, torch)
+        kernels["unpack_untilize_bfp8b_to_bf16_view_off_by_one_element_8x8192x8160"] = dict(ms=round(ms, 4), bytes=b, roofline=roofline("hbm", b / ms / 1e6, HBM_PEAK_GBS, "GB/s"))
+        del xv, pkv, backv
 
     # ---- Bfp8_b-weight GEMM and the FFN block --------------------------------------------------------
     gemm = {}

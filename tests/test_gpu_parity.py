@@ -219,6 +219,47 @@ def test_strided_and_unaligned_views_take_the_general_kernels(fmt):
             assert float(holder[:, :, :, 0::2].abs().sum()) == 0.0  # nothing written between the elements
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.uint16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("fmt", BFP + [F.Float16_b])
+def test_unit_stride_views_that_start_anywhere_stay_bit_exact(dtype, fmt):
+    """Sliced views of a row-major tensor (pybuda/pybuda/tensor.py:707-717): unit element stride, but a first element and a
+    row pitch that are multiples of the element size only.  They run on the row kernels (16-byte accesses that start
+    anywhere) and must give the bytes of the contiguous copy; on the way back nothing around the view may be touched."""
+    rng = np.random.default_rng(int(fmt) * 3 + (dtype == np.uint16))
+    tdt = torch.float32 if dtype == np.float32 else torch.bfloat16
+    # (holder columns, first column, columns): one element off; an odd row pitch; several segments with a partial last one
+    for width, c0, cols in ((192, 1, 160), (163, 2, 160), (1127, 3, 1120), (613, 7, 544)):
+        shape = (2, 2, 64, width)
+        base = make_input(rng, shape, "scaled", dtype)
+        view = base[:, :, :, c0:c0 + cols]
+        say("unaligned unit-stride view", fmt, dtype.__name__, width, c0, cols)
+        want = O.tilize_pack(np.ascontiguousarray(view), fmt)
+        dv = to_dev(base)[:, :, :, c0:c0 + cols]
+        assert dv.data_ptr() % 16 != 0 or (width * dv.element_size()) % 16 != 0
+        got = capi.tilize_pack(dv, fmt)
+        assert np.array_equal(to_np(got), want)
+        for dt, ofmt in ((torch.float32, F.Float32), (torch.bfloat16, F.Float16_b)):
+            want_rt = O.unpack_untilize(want, fmt, view.shape, ofmt)
+            holder = torch.full(shape, -77.0, dtype=dt, device=DEV)
+            capi.unpack_untilize(got, fmt, view.shape, out=holder[:, :, :, c0:c0 + cols])
+            assert np.array_equal(bits(to_np(holder[:, :, :, c0:c0 + cols].contiguous())), bits(want_rt))
+            assert bool((holder[:, :, :, :c0] == -77.0).all()) and bool((holder[:, :, :, c0 + cols:] == -77.0).all())
+        # ragged rows and columns of such a view: padding inside the pack launch, narrowing inside the unpack launch
+        rv, cv = 50, cols - 8
+        ragged = dv[:, :, :rv, :cv]
+        pad = np.zeros((2, 2, 64, cols), dtype=dtype)
+        pad[:, :, :rv, :cv] = view[:, :, :rv, :cv]
+        want_p = O.tilize_pack(pad, fmt)
+        got_p = capi.tilize_pack_padded(ragged, fmt)
+        assert np.array_equal(to_np(got_p), want_p)
+        holder = torch.full(shape, -77.0, dtype=tdt, device=DEV)
+        capi.unpack_untilize_narrow(got_p, fmt, (2, 2, rv, cv), out=holder[:, :, :rv, c0:c0 + cv])
+        want_n = O.unpack_untilize(want_p, fmt, (2, 2, 64, cols), F.Float32 if dtype == np.float32 else F.Float16_b)[:, :, :rv, :cv]
+        assert np.array_equal(bits(to_np(holder[:, :, :rv, c0:c0 + cv].contiguous())), bits(np.ascontiguousarray(want_n)))
+        holder[:, :, :rv, c0:c0 + cv] = -77.0
+        assert bool((holder == -77.0).all())
+
+
 def test_config1_bfp8_round_trip_1024():
     """fp32 [1,1,1024,1024] N(0,1) seed 0: packed bytes and round-trip floats bit-exact."""
     torch.manual_seed(0)

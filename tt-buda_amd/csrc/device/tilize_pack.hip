@@ -66,7 +66,8 @@ __device__ __forceinline__ void lds_store(uint8_t *p, uint64_t v)
 }
 
 // Fast path.  Requires: element stride == itemsize; base address and the three outer strides
-// multiples of 16 bytes; dst 16-byte aligned.  1-D grid of bands x segments with the segment index
+// multiples of the element size (a sliced view of a row-major tensor: its 16-byte loads then start anywhere); dst
+// 16-byte aligned.  1-D grid of bands x segments with the segment index
 // varying fastest, so that the workgroups resident at any moment sweep contiguous memory on both
 // sides instead of one column strip (which would camp on a few HBM channels).
 // QUEUE: the tiles go to their slots of a queue's per-core buffers instead of one linear run; a
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(256) void tilize_pack_rows(const uint8_t *__restric
         const uint8_t *col0 = src + w * g.s0 + z * g.s1 + (uint64_t)(in_cols ? c0 : g.Cl - EPL) * sizeof(SrcT);
         const uint32_t r0 = tr * kTile + wave * 8;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = load_stream(col0 + (uint64_t)min(r0 + i, g.Rl - 1) * g.s2);
+        for (int i = 0; i < 8; ++i) v[i] = load_stream_at<sizeof(SrcT)>(col0 + (uint64_t)min(r0 + i, g.Rl - 1) * g.s2);
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             if (!in_cols || (r0 + i >= g.Rl && !g.rep_r)) v[i] = make_uint4(0, 0, 0, 0);
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256) void tilize_pack_rows(const uint8_t *__restric
     const uint8_t *row0 = src + w * g.s0 + z * g.s1 + (uint64_t)(tr * kTile + wave * 8) * g.s2 +
                           (uint64_t)(live ? c0 : g.C - EPL) * sizeof(SrcT);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = load_stream(row0 + i * g.s2);
+    for (int i = 0; i < 8; ++i) v[i] = load_stream_at<sizeof(SrcT)>(row0 + i * g.s2);
     }
     if constexpr (QUEUE) {
         if (threadIdx.x < SEG_TILES && tile0 + threadIdx.x < tiles_c) tile_dst[threadIdx.x] = tile_offset(q, w, z, tr, tile0 + threadIdx.x);
@@ -346,8 +347,9 @@ hipError_t launch_kernel(const void *src, const TensorGeom &g, void *dst, const 
     const uint32_t tiles_r = g.R / kTile, tiles_c = g.C / kTile;
     const uint64_t bands = (uint64_t)g.W * g.Z * tiles_r;
     if (bands == 0 || tiles_c == 0) return hipSuccess;
-    const bool aligned = g.s3 == sizeof(SrcT) && ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) &&
-                         g.s0 % 16 == 0 && g.s1 % 16 == 0 && g.s2 % 16 == 0 && (!QUEUE || q.buffer_pitch % 16 == 0);
+    // unit element stride; the row-major side aligned to its elements (the strides are, by the boundary's checks), the tiles to 16 bytes
+    const bool aligned = g.s3 == sizeof(SrcT) && ((uintptr_t)src % sizeof(SrcT) == 0) && ((uintptr_t)dst % 16 == 0) &&
+                         (!QUEUE || q.buffer_pitch % 16 == 0);
     constexpr int SEG_TILES = 64 * Chunk<SrcT>::kElems / kTile;
     const uint32_t segs = (tiles_c + SEG_TILES - 1) / SEG_TILES;
     // padding on the fast path: whole chunks only, and a replicated column is a column of one element
