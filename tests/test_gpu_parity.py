@@ -416,13 +416,17 @@ def test_gemm_small_against_the_c_oracle():
                                    # K an odd number of tile rows (half a slab at the end) in every form of the macro-tiled kernel, and N an odd
                                    # number of tiles (the last tile column goes to one-row-tile workgroups of the weight-streaming kernel)
                                    (256, 96, 64), (256, 160, 128), (256, 288, 96), (4224, 96, 576), (3072, 160, 1024), (2176, 96, 2176),
-                                   (3072, 96, 4096), (768, 160, 16384), (416, 224, 224), (512, 4096, 4128), (512, 4128, 4096), (8192, 4128, 4128)])
+                                   (3072, 96, 4096), (768, 160, 16384), (416, 224, 224),
+                                   # 192 x 64 macro tiles with two pipelines (16 x 16 and 8 x 32 of them; the first above with half a slab
+                                   # at the end), and 128 x 128 with two pipelines where 192 does not divide M
+                                   (1536, 256, 2048), (3072, 128, 1024), (2048, 160, 1536), (2048, 256, 1536), (512, 4096, 4128), (512, 4128, 4096), (8192, 4128, 4128)])
 def test_gemm_kernel_selection_shapes(shape):
     """One shape per kernel path: one to four tile rows (weight streaming; K that splits unevenly over the wavefronts,
     fewer tile rows of W than wavefronts, slices of one, two, three and four whole tile pairs and of odd counts), ragged (general kernel), 128 x 64
     macro tiles (fewer than 256 tiles of 128 x 128; up to 256 of them in the form with rings - one pipeline where K is an odd number of slabs:
     one, three; two pipelines else: one slab each, two, three; N = 64, N a multiple of 64 only - more in the two-stage form: 33 x 8 tiles),
-    128 x 128 macro tiles with two pipelines (16 x 9 and 8 x 32 of them, two slabs and one slab per pipeline), 384 x 128 macro tiles
+    128 x 128 macro tiles with two pipelines (16 x 9 and 8 x 32 of them, two slabs and one slab per pipeline), 192 x 64 macro tiles with
+    two pipelines, 384 x 128 macro tiles
     (8 x 32 and 16 x 16 of them, where they fill the CUs better than 256 x 256: three slabs, one slab), 128 x 128 macro tiles (17 x 17 of them), and
     enough tiles for the 256 x 256 macro tiles (M = 768); all against
     dequantize-then-fp32-matmul with bias and GELU in both of the reference's forms."""

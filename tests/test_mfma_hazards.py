@@ -22,7 +22,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DEVICE = os.path.join(ROOT, "tt-buda_amd", "csrc", "device")
 # the 8-wave kernel, the 4-wave kernel with the narrow tile, and the panel form with its three LDS stages
-UNITS = ["gemm_bfp8b_big_bf16.hip", "gemm_bfp8b_slim_f32.hip", "gemm_bfp8b_panel_small_bf16.hip", "gemm_bfp8b_duo_slim_bf16.hip", "gemm_bfp8b_duo_small_f32.hip", "gemm_bfp8b_tall_bf16.hip"]
+UNITS = ["gemm_bfp8b_big_bf16.hip", "gemm_bfp8b_slim_f32.hip", "gemm_bfp8b_panel_small_bf16.hip", "gemm_bfp8b_duo_slim_bf16.hip", "gemm_bfp8b_duo_small_f32.hip", "gemm_bfp8b_tall_bf16.hip", "gemm_bfp8b_duo_lean_bf16.hip"]
 
 
 def build_flags():

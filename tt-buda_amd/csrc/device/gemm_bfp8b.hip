@@ -58,7 +58,7 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn,
     //   else at most one 128 x 128 workgroup per CU: that tile on two stages with two pipelines (K a multiple of 128) -
     //     3072 x 1024 x 4096: 44.5 us against 53 for 384 workgroups of 128 x 64, 512 x 8192 x 2048: 29 against 33;
     //   else 128 x 64 on two stages below 256 tiles of 128 x 128 (three workgroups fit a CU), 128 x 128 above.
-    // TTBFP_GEMM_TILE (1: 128 x 64 on two stages, 2: 128 x 128 on two stages, 3: 256 x 256 where it fits, 5: 384 x 128 where it fits) and
+    // TTBFP_GEMM_TILE (1: 128 x 64 on two stages, 2: 128 x 128 on two stages, 3: 256 x 256 where it fits, 5: 384 x 128 where it fits, 6: 192 x 64 with two pipelines where it fits) and
     // TTBFP_GEMM_PIPELINES=1 (no workgroup with two pipelines) are tuning aids for measurements and override this.
     const int force = force_tile();
     static const bool duo = [] { const char *v = getenv("TTBFP_GEMM_PIPELINES"); return !v || atoi(v) != 1; }();
@@ -70,6 +70,13 @@ static hipError_t launch_tiled(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn,
         return f32 ? launch_gemm_bfp8b_ring_slim_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_ring_slim_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     }
+    // 192 x 64 tiles with two pipelines where they give more workgroups than 128 x 128 tiles and still at most one per CU
+    // (3072 x 1024 x 4096: 256 against 192)
+    const uint64_t lean_tiles = (uint64_t)(M / 192) * (N / 64);
+    if ((force == 0 || force == 6) && duo && gemm_fits<LeanShape>(M, N, K) && (K / 64) % 2 == 0 && lean_tiles <= TTBFP_CUS &&
+        (force == 6 || (slim_tiles > TTBFP_CUS && lean_tiles > small_tiles)))
+        return f32 ? launch_gemm_bfp8b_duo_lean_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
+                   : launch_gemm_bfp8b_duo_lean_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);
     if (force == 0 && duo && gemm_fits<SmallShape>(M, N, K) && small_tiles <= TTBFP_CUS && (K / 64) % 2 == 0)
         return f32 ? launch_gemm_bfp8b_duo_small_f32(M, N, K, ldn, x, w, bias, epilogue, y, stream)
                    : launch_gemm_bfp8b_duo_small_bf16(M, N, K, ldn, x, w, bias, epilogue, y, stream);

@@ -309,7 +309,8 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     constexpr int BM = S::BM, BN = S::BN, MB = S::MB, NB = S::NB, XI = S::XI, PW = S::PW, KH = S::KH;
     constexpr uint32_t A_BYTES = S::A_BYTES, STAGE = S::STAGE;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
-    static_assert(GROUPS == 1 || (GROUPS == 2 && S::NW == 4 && !PANEL && !SPLITK && (MB * NB) % 2 == 0), "two pipelines: packed W, four wavefronts each");
+    // (an odd number of blocks per wavefront is split unevenly at the end: pipeline 0 finishes the even ones, one more)
+    static_assert(GROUPS == 1 || (GROUPS == 2 && S::NW == 4 && !PANEL && !SPLITK && MB * NB >= 2), "two pipelines: packed W, four wavefronts each");
     const uint32_t group = GROUPS == 1 ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x / S::NT);  // pipeline of this wavefront
     uint8_t *const lds = lds_all + group * pipeline_lds_bytes<S, PANEL, RING>();
 
@@ -841,12 +842,16 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     constexpr uint32_t PITCH = kImagePitch<S>;
     uint8_t *const image = lds_all + exchange_lds_bytes<S, GROUPS>();
     if constexpr (STAGED && GROUPS == 1) __syncthreads();  // every wavefront has read its last operands (two pipelines: the barriers above)
+    // The activation is chosen once for the whole tile, not per element: straight-line code lets the compiler interleave the
+    // independent chains of a lane's values (a reciprocal and an exponential each) instead of finishing them one by one.
+    auto finish_blocks = [&](auto actc) {
+    constexpr int ACTIVATION = decltype(actc)::value;
     auto finished = [&](auto bc, auto rc, float bv) {  // element r of block BLK with bias and activation applied
         constexpr int BLK = decltype(bc)::value, r = decltype(rc)::value;
         float v = accumulator_read<16 * BLK + r, ALL_AGPRS>();
         if constexpr (GROUPS == 2) v += *exchange_at(BLK, r);
         v += bv;
-        return apply_epilogue(epilogue & kEpilogueMask, v);  // uniform branches
+        return apply_epilogue(ACTIVATION, v);
     };
     static_for<MB * NB>([&](auto bc) {
         constexpr int BLK = decltype(bc)::value, mb = BLK / NB, nb = BLK % NB;
@@ -872,6 +877,12 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
             });
         }
     });
+    };
+    switch (epilogue & kEpilogueMask) {  // uniform
+        case 1: finish_blocks(integral_constant<int, 1>{}); break;
+        case 2: finish_blocks(integral_constant<int, 2>{}); break;
+        default: finish_blocks(integral_constant<int, 0>{}); break;
+    }
     if constexpr (STAGED) {
         __syncthreads();
         constexpr int LPR = BN * 2 / 16;                // lanes per row of the tile: 16 bytes each
@@ -982,6 +993,10 @@ using SlimShape = Shape<128, 64, 2, 2>;
 // 256 x 256 tiles give 192.  Eight wavefronts, wave tile 96 x 64 (five operand reads for the six MFMAs of a k step; as 192 x 32
 // it would be seven: 3072 x 4096 x 4096 94-97 against 98-103 us).
 using TallShape = Shape<384, 128, 4, 2>;
+// One and a half tile rows of 128, half the width: M = 3072 at N = 1024 gives 16 x 16 = 256 workgroups, one per CU, where 128 x 128
+// tiles give 192.  Four wavefronts 2 x 2 (wave tile 96 x 32), two pipelines per workgroup: a thread dequantizes 16 weights
+// per slab for the wavefront's 12 MFMAs, where the 128 x 128 tile has 32 for 16.
+using LeanShape = Shape<192, 64, 2, 2>;
 
 // true if the problem can be cut into macro tiles of shape S
 template <typename S>
@@ -1008,6 +1023,8 @@ TTBFP_DECLARE_GEMM(duo_slim_f32);  // SlimShape in the ring form, two pipelines 
 TTBFP_DECLARE_GEMM(duo_slim_bf16);
 TTBFP_DECLARE_GEMM(duo_small_f32);  // SmallShape on two stages, two pipelines per workgroup
 TTBFP_DECLARE_GEMM(duo_small_bf16);
+TTBFP_DECLARE_GEMM(duo_lean_f32);  // LeanShape on two stages, two pipelines per workgroup
+TTBFP_DECLARE_GEMM(duo_lean_bf16);
 TTBFP_DECLARE_GEMM(panel_f32);   // BigShape on a bf16 panel of W instead of the packed tiles
 TTBFP_DECLARE_GEMM(panel_bf16);
 TTBFP_DECLARE_GEMM(panel_small_f32);  // SmallShape on a panel made for 128-wide tiles
