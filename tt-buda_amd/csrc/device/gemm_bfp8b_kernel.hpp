@@ -846,35 +846,35 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     // independent chains of a lane's values (a reciprocal and an exponential each) instead of finishing them one by one.
     auto finish_blocks = [&](auto actc) {
     constexpr int ACTIVATION = decltype(actc)::value;
-    auto finished = [&](auto bc, auto rc, float bv) {  // element r of block BLK with bias and activation applied
-        constexpr int BLK = decltype(bc)::value, r = decltype(rc)::value;
-        float v = accumulator_read<16 * BLK + r, ALL_AGPRS>();
-        if constexpr (GROUPS == 2) v += *exchange_at(BLK, r);
-        v += bv;
-        return apply_epilogue(ACTIVATION, v);
-    };
     static_for<MB * NB>([&](auto bc) {
         constexpr int BLK = decltype(bc)::value, mb = BLK / NB, nb = BLK % NB;
         if (GROUPS == 2 && (BLK & 1) != (int)group) return;
         const uint32_t col_in_tile = wn * (BN / S::WN) + nb * 32 + (lane & 31);
         const uint32_t row_in_tile = wm * (BM / S::WM) + mb * 32 + (lane >> 5) * 4;
         const float bv = bias ? load_bias(bias, n0 + col_in_tile, epilogue & kEpilogueBiasF32) : 0.0f;
+        // The block's sixteen values leave the accumulators first (statements the compiler keeps in order), then bias and
+        // activation are applied to all of them in ordinary code: sixteen independent chains to interleave.
+        float v[16];
+        static_for<16>([&](auto rc) { v[decltype(rc)::value] = accumulator_read<16 * BLK + decltype(rc)::value, ALL_AGPRS>(); });
+        if constexpr (GROUPS == 2) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) v[r] += *exchange_at(BLK, r);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = apply_epilogue(ACTIVATION, v[r] + bv);
         if constexpr (STAGED) {
             uint8_t *ip = image + row_in_tile * PITCH + col_in_tile * 2;
-            static_for<8>([&](auto pc) {
-                constexpr int r0 = 2 * decltype(pc)::value, r1 = r0 + 1;
-                constexpr uint32_t rr0 = (r0 >> 2) * 8 + (r0 & 3), rr1 = (r1 >> 2) * 8 + (r1 & 3);  // rows inside the block, before the lane's 4-row offset
-                const uint32_t pair = pack_bf16_rne(finished(bc, integral_constant<int, r0>{}, bv), finished(bc, integral_constant<int, r1>{}, bv));
+#pragma unroll
+            for (int r0 = 0; r0 < 16; r0 += 2) {
+                const uint32_t rr0 = (r0 >> 2) * 8 + (r0 & 3), rr1 = rr0 + 1;  // rows inside the block, before the lane's 4-row offset
+                const uint32_t pair = pack_bf16_rne(v[r0], v[r0 + 1]);
                 *(uint16_t *)(ip + rr0 * PITCH) = (uint16_t)pair;
                 *(uint16_t *)(ip + rr1 * PITCH) = (uint16_t)(pair >> 16);
-            });
+            }
         } else {
             OutT *yp = Y + (uint64_t)(m0 + row_in_tile) * ldn + n0 + col_in_tile;
-            static_for<16>([&](auto rc) {
-                constexpr int r = decltype(rc)::value;
-                constexpr uint32_t rr = (r >> 2) * 8 + (r & 3);
-                yp[(uint64_t)rr * ldn] = finished(bc, rc, bv);
-            });
+#pragma unroll
+            for (int r = 0; r < 16; ++r) yp[(uint64_t)((r >> 2) * 8 + (r & 3)) * ldn] = v[r];
         }
     });
     };
