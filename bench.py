@@ -57,6 +57,14 @@ def parse():
     p.add_argument("--sustained-seconds", type=float, default=2.0,
                    help="length of the sustained 8192^3 loops whose clock and power are sampled (0: skip them)")
     p.add_argument("--no-host-push", action="store_true", help="skip the host push / read-back lines (PCIe inclusive)")
+    p.add_argument("--ablation", action="store_true",
+                   help="instead of the benchmark: time the fused 8192^3 GEMM of the library and of every tt-buda_amd/libttbfp_ablate<bits>.so "
+                        "beside it (make -C tt-buda_amd/csrc ablate ABLATE=<bits>: parts of the kernel's work left out, wrong results on purpose), "
+                        "each in a sustained loop with clock and power sampled; prints one JSON line")
+    p.add_argument("--data-probe", action="store_true",
+                   help="instead of the benchmark: the fused 8192^3 GEMM on random, constant and all-zero operands, each in a sustained loop "
+                        "with clock and power sampled (the kernel's cycle count does not depend on the data; the clock the power cap allows does); "
+                        "prints one JSON line")
     p.add_argument("--power-probe", type=float, default=0.0, metavar="SECONDS",
                    help="instead of the benchmark: run each 8192^3 GEMM form (fused, with workspace, the vendor library's plain bf16 "
                         "GEMM through torch.matmul) back to back for SECONDS while rocm-smi is polled for clock and power; prints one JSON line")
@@ -178,6 +186,57 @@ def sustained(fn, seconds, flops, torch):
             # what the matrix cores deliver at the clock the part ran at: 256 CUs x 4 SIMDs x 1024 flop per clock
             "mfma_peak_at_clock_tflops": round(256 * 4 * 1024 * clock * 1e6 / 1e12, 1) if clock else None,
             "frac_of_peak_at_clock": round(tf / (256 * 4 * 1024 * clock * 1e6 / 1e12), 4) if clock else None}
+
+
+def ablation_probe(seconds, torch, capi):
+    """What the parts of the 256 x 256 kernel cost: the same 8192^3 launch from the library and from its ablated copies."""
+    import ctypes
+    import glob
+
+    F = capi.DataFormatCode
+    n = 8192
+    g = torch.Generator(device="cuda:0").manual_seed(30)
+    wp = capi.tilize_pack(torch.randn(1, 1, n, n, generator=g, device="cuda:0") * 0.02, F.Bfp8_b)
+    g = torch.Generator(device="cuda:0").manual_seed(31)
+    x = torch.randn(n, n, generator=g, device="cuda:0").bfloat16()
+    y = torch.empty(n, n, dtype=torch.bfloat16, device="cuda:0")
+    left_out = {1: "dequantization", 2: "X loads", 4: "W fetches", 8: "MFMAs"}
+    libs = [("the library (nothing left out)", capi.lib())]
+    for path in sorted(glob.glob(os.path.join(os.path.dirname(capi.LIB_PATH), "libttbfp_ablate*.so"))):
+        bits = int(os.path.basename(path)[len("libttbfp_ablate"):-3])
+        L = ctypes.CDLL(path)
+        L.ttbfp_gemm_bfp8b_bf16.restype, L.ttbfp_gemm_bfp8b_bf16.argtypes = capi.SYMBOLS["ttbfp_gemm_bfp8b_bf16"]
+        libs.append(("without " + ", ".join(v for k, v in left_out.items() if bits & k) + " (TTBFP_ABLATE=%d)" % bits, L))
+    out = {}
+    for name, L in libs:
+        def fn(L=L):
+            st = L.ttbfp_gemm_bfp8b_bf16(n, n, n, x.data_ptr(), wp.data_ptr(), None, 0, y.data_ptr(), F.Float16_b, capi._stream())
+            assert st == 0
+        out[name] = sustained(fn, seconds, 2.0 * n ** 3, torch)
+    print(json.dumps({"ablation_seconds": seconds, "shape": "8192 x 8192 x 8192, fused kernel on 256 x 256 tiles, bf16 result", "forms": out}))
+
+
+def data_probe(seconds, torch, capi):
+    """The same launch on operands that make the matrix cores switch more or fewer bits: what the power cap costs."""
+    F = capi.DataFormatCode
+    n = 8192
+    g = torch.Generator(device="cuda:0").manual_seed(30)
+    w_rand = capi.tilize_pack(torch.randn(1, 1, n, n, generator=g, device="cuda:0") * 0.02, F.Bfp8_b)
+    g = torch.Generator(device="cuda:0").manual_seed(31)
+    x_rand = torch.randn(n, n, generator=g, device="cuda:0").bfloat16()
+    w_const = capi.tilize_pack(torch.full((1, 1, n, n), 0.0123, device="cuda:0"), F.Bfp8_b)
+    w_zero = torch.zeros_like(w_rand)
+    x_zero = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda:0")
+    y = torch.empty(n, n, dtype=torch.bfloat16, device="cuda:0")
+    cases = [("W N(0,0.02), X N(0,1): the benchmark's operands", w_rand, x_rand), ("W one value (0.0123), X N(0,1)", w_const, x_rand),
+             ("W all-zero tiles, X N(0,1)", w_zero, x_rand), ("W N(0,0.02), X zero", w_rand, x_zero), ("W zero, X zero", w_zero, x_zero)]
+    out = {}
+    for name, wp, x in cases:
+        r = sustained(lambda: capi.gemm_bfp8b(x, wp, n, out=y), seconds, 2.0 * n ** 3, torch)
+        if r["clock_mhz"]:
+            r["cycles_per_simd"] = round(r["ms"] * 1e-3 * r["clock_mhz"] * 1e6)
+        out[name] = r
+    print(json.dumps({"data_probe_seconds": seconds, "shape": "8192 x 8192 x 8192, fused kernel, bf16 result", "forms": out}))
 
 
 def time_kernel(fn, steps, warmup, torch):
@@ -310,6 +369,12 @@ def main():
     dev = "cuda:0"
     if args.power_probe > 0:
         power_probe(args.power_probe, torch, capi)
+        return
+    if args.ablation:
+        ablation_probe(args.sustained_seconds or 2.0, torch, capi)
+        return
+    if args.data_probe:
+        data_probe(args.sustained_seconds or 2.0, torch, capi)
         return
 
     # ---- streaming workload: bf16 [8,1,8192,8192], U(-8,8), seed 2 --------------------------------

@@ -51,6 +51,15 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int BK = 64;
 constexpr int A_ROW = BK * 2;  // bytes per A row in LDS
+
+// Measurement aid, never set in the library that ships (make -C tt-buda_amd/csrc ablate ABLATE=<bits> builds a copy of the
+// library whose 256 x 256 kernel leaves parts of its work out, for bench.py --ablation to time): bit 0 no dequantization (the
+// B stage is never written), bit 1 no X loads, bit 2 no W fetches (the dequantization then runs on whatever the registers
+// hold, kept alive as opaque values), bit 3 no MFMAs, bit 4 the dequantization without its LDS stores.  The results of such
+// a build are garbage; what it shows is what the rest of the kernel costs.
+#ifndef TTBFP_ABLATE
+#define TTBFP_ABLATE 0
+#endif
 constexpr uint32_t kW8Tile = tile_bytes(kBfp8_b);
 
 // Where column n of a B stage sits inside its group of eight columns: slot (n & 7) ^ key(n / 8).  A 128-bit operand read
@@ -99,9 +108,12 @@ __device__ __forceinline__ void static_for(F &&f)
 }
 
 // Shape of one workgroup: BM x BN macro tile, WM x WN wavefronts (each owns BM/WM x BN/WN).
-template <int BM_, int BN_, int WM_, int WN_>
+template <int BM_, int BN_, int WM_, int WN_, bool WDIRECT_ = false>
 struct Shape {
     static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+    // the data sections of W's tiles travel by direct loads into raw areas of LDS (two-stage form; see the kernel)
+    static constexpr bool WDIRECT = WDIRECT_;
+    static constexpr uint32_t RAW_BYTES = WDIRECT_ ? (uint32_t)(2 * (BN_ / 32) * 1024) : 0u;  // the data of a slab's tiles
     static constexpr int NW = WM * WN, NT = 64 * NW;            // wavefronts, threads
     static constexpr int MB = BM / WM / 32, NB = BN / WN / 32;  // 32x32 blocks per wave in m and n
     static constexpr int XI = BM / 8 / NW;                      // direct X loads (8 rows each) per wave per slab
@@ -154,6 +166,7 @@ struct Shape {
 template <int IDX, bool GUARD, bool ALL>
 __device__ __forceinline__ void mfma_accumulate(const bf16x8 &a, const bf16x8 &b)
 {
+    if constexpr ((TTBFP_ABLATE & 8) != 0) return;
 #define TTBFP_MFMA_INS "v"(a), "v"(b), "n"(16 * IDX), "n"(16 * IDX + 15)
     if constexpr (GUARD)
         TTBFP_ACC_ASM(ALL, "s_nop 1\n\tv_mfma_f32_32x32x16_bf16 a[%c2:%c3], %0, %1, a[%c2:%c3]", , TTBFP_MFMA_INS);
@@ -247,7 +260,7 @@ constexpr uint32_t pipeline_lds_bytes()
     if constexpr (RING > 0)
         return ring_lds_bytes<S, RING>();
     else
-        return (PANEL ? panel_stages<S>() : 2) * S::STAGE;
+        return (PANEL ? panel_stages<S>() : 2) * S::STAGE + (PANEL ? 0u : 2 * S::RAW_BYTES);
 }
 
 // Bytes that the two pipelines of a workgroup exchange their partial sums through (0 with one pipeline)
@@ -366,6 +379,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     }
     auto load_x = [&](uint32_t slab, uint32_t stage, auto ic) {
         constexpr int I = decltype(ic)::value;
+        if constexpr ((TTBFP_ABLATE & 2) != 0) return;
         direct_load_16<(I % 4) * 1024>(x_wave + (uint64_t)slab * (BK * 2), x_off[I],
                                                    lds_base + stage * STAGE + (wave * XI + I / 4 * 4) * 8 * A_ROW);
     };
@@ -393,9 +407,20 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     // Two register sets, set q holding slabs of parity q: while one is dequantized into LDS the loads
     // of the following slab are in flight into the other, a whole iteration ahead of their use.
     WPatch<PW, KH> wp[2];
+    if constexpr ((TTBFP_ABLATE & 4) != 0) {  // never fetched: values the optimizer cannot see through
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            wp[q].e = make_uint2(opaque(0x78797a7bu), opaque(0x7a797877u));
+#pragma unroll
+            for (int j = 0; j < KH; ++j)
+#pragma unroll
+                for (int c = 0; c < PW / 4; ++c) wp[q].d[j][c] = opaque(0x01020304u * (j + 1) + lane);
+        }
+    }
     constexpr int WU = 1 + KH;  // fetch units per slab
     auto fetch_w = [&](uint32_t slab, auto pc, auto uc) {  // unit 0: exponents, units 1..KH: datum rows
         constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
+        if constexpr ((TTBFP_ABLATE & 4) != 0) return;
         const uint8_t *t = w_src + slab * w_slab_bytes;
         if constexpr (U == 0 && KH == 4) {
             wp[P].e.x = *(const uint32_t *)(t + w_face * 16 + w_kh * 8 + w_half * 4);
@@ -408,6 +433,41 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         } else {
             wp[P].d[U - 1][0] = *(const uint32_t *)(t + kExpSection + w_in_tile + (U - 1) * 16);
         }
+    };
+
+    // WDIRECT (two-stage form): a thread's patch is eight 4-byte pieces of eight different 16-byte face rows, so fetched
+    // into registers a wavefront's load touches sixteen cache lines for 256 bytes, nine loads per slab.  Instead the
+    // 1024-byte data section of every tile of the slab goes into a raw area of LDS by ONE direct load (64 lanes x 16
+    // bytes, contiguous in memory), slab s + 3 during iteration s, and the threads pick their patches out of it with
+    // 4-byte LDS reads at the start of iteration s + 1; only the exponent bytes still travel through registers.  Two raw
+    // areas: the one slab s + 3 lands in was last read at the start of iteration s, before the barrier at its end.
+    // Inside a tile's image the 16-byte rows are permuted, row c stored at c ^ (tile column & 7): a patch read takes the
+    // same row of sixteen (tile, face) pairs, which would all sit on four banks otherwise.
+    constexpr bool WDIRECT = S::WDIRECT && !PANEL && !SPLITK && RING == 0;
+    constexpr uint32_t RAWD = S::RAW_BYTES, RAWD_BASE = 2 * STAGE;
+    constexpr int WT = WDIRECT ? 2 * (BN / kTile) / S::NW : 1;  // tiles (direct loads) per wavefront and slab
+    static_assert(!WDIRECT || (2 * (BN / kTile)) % S::NW == 0, "whole tiles per wavefront");
+    static_assert(!WDIRECT || PW == 4, "a thread's patch: rows of one dword");
+    uint32_t wd_off[WT];  // lane's offset from the first tile of the slab's first tile row: tile, data section, permuted row
+#pragma unroll
+    for (int i = 0; i < WT; ++i) {
+        const uint32_t ti = wave * WT + i, tr = ti / (BN / kTile), tc = ti % (BN / kTile);
+        wd_off[i] = (tr * tiles_n + tc) * kW8Tile + kExpSection + ((lane ^ (tc & 7u)) * 16);
+    }
+    const uint64_t wd_base = uniform64((uint64_t)(uintptr_t)Wp + (uint64_t)(n0 / kTile) * kW8Tile + (uint64_t)split * nslabs * w_slab_bytes);
+    auto load_w_direct = [&](uint32_t slab, uint32_t area, auto ic) {
+        constexpr int I = decltype(ic)::value;
+        if constexpr ((TTBFP_ABLATE & 4) != 0) return;
+        direct_load_16<0>(wd_base + (uint64_t)slab * w_slab_bytes, wd_off[I], lds_base + RAWD_BASE + area * RAWD + (wave * WT + I) * 1024);
+    };
+    // this thread's patch inside a raw area: tile (tile row of the slab, tile column), row group of eight, quarter of a row
+    // (rows w_half * 4 + U - 1 of the group of eight; the permutation key and the half are folded into the address, the unit is XORed in)
+    const uint32_t wd_patch = RAWD_BASE + ((w_kc >> 2) * (BN / kTile) + w_n / kTile) * 1024 + (w_face * 16 + w_kh * 8) * 16 + (w_n & 12u) +
+                              ((((w_n / kTile) & 7u) ^ (w_half * 4)) << 4);
+    auto read_w_direct = [&](uint32_t area, auto pc, auto uc) {  // unit U = 1 .. 8: row U - 1 of the patch
+        constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
+        if constexpr ((TTBFP_ABLATE & 4) != 0) return;
+        wp[P].d[U - 1][0] = *(const uint32_t *)(lds + area * RAWD + (wd_patch ^ ((U - 1) << 4)));
     };
 
     // ---- staging of a W register set into an LDS stage, cut into small units ----------------------
@@ -433,6 +493,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     uint32_t q_sgn[2], q_mag;
     auto dequant_step = [&](uint8_t *st, auto pc, auto uc) {
         constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
+        if constexpr ((TTBFP_ABLATE & 1) != 0) return;
         constexpr int G = U / 4, MS = U % 4, I = G / (KH / 4), H = G % (KH / 4), C = I / 4, B = I % 4, R = 4 * H;
         constexpr uint32_t SIGN_SEL = 0x000c000cu | ((uint32_t)(4 + B) << 24) | ((uint32_t)B << 8);
         if constexpr (MS == 0) {
@@ -455,7 +516,9 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
             const uint32_t mag1 = __builtin_amdgcn_perm(__float_as_uint(q_f[3]), __float_as_uint(q_f[2]), 0x07060302u);
             w_col[2 * H] = (q_sgn[0] & 0x80008000u) | q_mag;
             w_col[2 * H + 1] = (q_sgn[1] & 0x80008000u) | mag1;
-            if constexpr (KH == 4)  // this thread's four k of the column
+            if constexpr ((TTBFP_ABLATE & 16) != 0) {  // computed, not stored
+                asm volatile("" : : "v"(w_col[2 * H]), "v"(w_col[2 * H + 1]));
+            } else if constexpr (KH == 4)  // this thread's four k of the column
                 *(uint2 *)(st + w_lds + ((((w_n & 7u) + I) ^ w_key) * 16)) = make_uint2(w_col[0], w_col[1]);
             else if constexpr (H == 1)  // the column is complete: store its eight k as one 128-bit vector
                 *(uint4 *)(st + w_lds + ((((w_n & 7u) + I) ^ w_key) * 16)) = make_uint4(w_col[0], w_col[1], w_col[2], w_col[3]);
@@ -575,6 +638,8 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     constexpr int X_STEP = (SLOTS / 2 - X_FIRST) / XI > 1 ? (SLOTS / 2 - X_FIRST) / XI : 1;
     static_assert(X_FIRST + (XI - 1) * X_STEP < SLOTS, "every X load needs a slot");
     static_assert(WU <= SLOTS, "every W fetch needs a slot");
+    constexpr int XW_STEP = (SLOTS - 1 - WT) / XI >= 2 ? 2 : 1;  // slots between the X loads of the WDIRECT form
+    static_assert(!WDIRECT || 1 + WT + (XI - 1) * XW_STEP < SLOTS, "every direct load needs a slot");
 
     // One iteration (P = s & 1): the last AHEAD k steps of slab s, then the first 4 - AHEAD of slab s+1 (stage P^1).
     // With STAGING, slab s+2 is assembled in stage P meanwhile and a barrier publishes it at the end.
@@ -590,7 +655,24 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
             k_step(integral_constant<int, ((G + 4 - AHEAD) % 4) % NBUF>{}, [&](auto uc) {
                 constexpr int U = decltype(uc)::value, T = G * MF + U;
                 if constexpr (U < MB + NB) read_frag(cur, uc, integral_constant<int, G>{}, integral_constant<int, G % NBUF>{});
-                if constexpr (STAGING) {
+                if constexpr (STAGING && WDIRECT) {
+                    if constexpr (T == 0) {
+                        // the patch of slab s + 2 out of its raw area (it landed before the barrier that ended iteration s - 1),
+                        // the exponents of slab s + 3 into the other register set
+                        static_for<KH>([&](auto jc) { read_w_direct(P, pc, integral_constant<int, 1 + decltype(jc)::value>{}); });
+                        fetch_w(w_slab, integral_constant<int, P ^ 1>{}, integral_constant<int, 0>{});
+                        stage_exponents(pc);
+                    }
+                    static_for<WT>([&](auto ic) {  // the data of slab s + 3 into the raw area slab s + 1 was read from an iteration ago
+                        if constexpr (1 + decltype(ic)::value == T) load_w_direct(w_slab, P ^ 1, ic);
+                    });
+                    static_for<NU>([&](auto kc) {  // micro-steps spread evenly over slots 2 .. SLOTS - 1: the patch reads have had a slot to land
+                        if constexpr (2 + decltype(kc)::value * (SLOTS - 2) / NU == T) dequant_step(dst, pc, kc);
+                    });
+                    static_for<XI>([&](auto ic) {
+                        if constexpr (1 + WT + decltype(ic)::value * XW_STEP == T) load_x(s + 2, P, ic);
+                    });
+                } else if constexpr (STAGING) {
                     if constexpr (T < WU) fetch_w(w_slab, integral_constant<int, P ^ 1>{}, integral_constant<int, T>{});
                     if constexpr (T == 0) stage_exponents(pc);
                     static_for<NU>([&](auto kc) {  // micro-steps spread evenly over slots 1 .. SLOTS - 1
@@ -746,7 +828,12 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     static_for<XI>([&](auto ic) { load_x(last < 1 ? last : 1, 1, ic); });
     stage_exponents(P1);
     static_for<NU>([&](auto kc) { dequant_step(lds + STAGE, P1, kc); });
-    static_for<WU>([&](auto uc) { fetch_w(last < 2 ? last : 2, P0, uc); });
+    if constexpr (WDIRECT) {  // slab 2: its exponents into register set 0, its data into raw area 0
+        fetch_w(last < 2 ? last : 2, P0, integral_constant<int, 0>{});
+        static_for<WT>([&](auto ic) { load_w_direct(last < 2 ? last : 2, 0, ic); });
+    } else {
+        static_for<WU>([&](auto uc) { fetch_w(last < 2 ? last : 2, P0, uc); });
+    }
     }
     wait_direct_loads();
     __syncthreads();
@@ -981,8 +1068,11 @@ hipError_t launch_shape(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const 
 
 // The macro-tile shapes in use.  Each (shape, output type) pair is compiled in a translation unit
 // of its own (gemm_bfp8b_<shape>_<type>.hip) so that the build can run them in parallel.
+#ifndef TTBFP_BIG_WDIRECT
+#define TTBFP_BIG_WDIRECT true
+#endif
 #ifndef TTBFP_BIG_SHAPE
-#define TTBFP_BIG_SHAPE Shape<256, 256, 2, 4>
+#define TTBFP_BIG_SHAPE Shape<256, 256, 2, 4, TTBFP_BIG_WDIRECT>
 #endif
 using BigShape = TTBFP_BIG_SHAPE;
 using SmallShape = Shape<128, 128, 2, 2>;
