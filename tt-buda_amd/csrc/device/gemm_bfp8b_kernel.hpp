@@ -441,8 +441,9 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     // bytes, contiguous in memory), slab s + 3 during iteration s, and the threads pick their patches out of it with
     // 4-byte LDS reads at the start of iteration s + 1; only the exponent bytes still travel through registers.  Two raw
     // areas: the one slab s + 3 lands in was last read at the start of iteration s, before the barrier at its end.
-    // Inside a tile's image the 16-byte rows are permuted, row c stored at c ^ (tile column & 7): a patch read takes the
-    // same row of sixteen (tile, face) pairs, which would all sit on four banks otherwise.
+    // Inside a tile's image the 16-byte rows are permuted, row c stored at c ^ key with key = 2 (tile column & 3) + (face & 1):
+    // a patch read takes the same row of sixteen (tile, face) pairs, which would all sit on four banks otherwise; the
+    // eight pairs of a half-wavefront get eight different keys.
     constexpr bool WDIRECT = S::WDIRECT && !PANEL && !SPLITK && RING == 0;
     constexpr uint32_t RAWD = S::RAW_BYTES, RAWD_BASE = 2 * STAGE;
     constexpr int WT = WDIRECT ? 2 * (BN / kTile) / S::NW : 1;  // tiles (direct loads) per wavefront and slab
@@ -452,7 +453,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
 #pragma unroll
     for (int i = 0; i < WT; ++i) {
         const uint32_t ti = wave * WT + i, tr = ti / (BN / kTile), tc = ti % (BN / kTile);
-        wd_off[i] = (tr * tiles_n + tc) * kW8Tile + kExpSection + ((lane ^ (tc & 7u)) * 16);
+        wd_off[i] = (tr * tiles_n + tc) * kW8Tile + kExpSection + ((lane ^ (((tc & 3u) << 1) | ((lane >> 4) & 1u))) * 16);
     }
     const uint64_t wd_base = uniform64((uint64_t)(uintptr_t)Wp + (uint64_t)(n0 / kTile) * kW8Tile + (uint64_t)split * nslabs * w_slab_bytes);
     auto load_w_direct = [&](uint32_t slab, uint32_t area, auto ic) {
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     // this thread's patch inside a raw area: tile (tile row of the slab, tile column), row group of eight, quarter of a row
     // (rows w_half * 4 + U - 1 of the group of eight; the permutation key and the half are folded into the address, the unit is XORed in)
     const uint32_t wd_patch = RAWD_BASE + ((w_kc >> 2) * (BN / kTile) + w_n / kTile) * 1024 + (w_face * 16 + w_kh * 8) * 16 + (w_n & 12u) +
-                              ((((w_n / kTile) & 7u) ^ (w_half * 4)) << 4);
+                              ((((((w_n / kTile) & 3u) << 1) | (w_face & 1u)) ^ (w_half * 4)) << 4);
     auto read_w_direct = [&](uint32_t area, auto pc, auto uc) {  // unit U = 1 .. 8: row U - 1 of the patch
         constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
         if constexpr ((TTBFP_ABLATE & 4) != 0) return;
