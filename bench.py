@@ -29,20 +29,20 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # factor 1.0).  Summary: profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES = {
     # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) x 1024 per launch; the two factors come from the 1 GiB copy in the same runs
-    "tilize_pack": 1644307484,      # 1,644,167,168 algorithmic
-    "unpack_untilize": 1644374071,
+    "tilize_pack": 1644306288,      # 1,644,167,168 algorithmic
+    "unpack_untilize": 1644385769,
     # GEMM kernels, same method: profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt (the forms with a workspace include
     # their first pass / their reduction; the FFN figure is the sum of its two matmuls)
-    "gemm_8192": 1242390816, "gemm_8192_ws": 1954445758, "gemm_M8192": 344673778, "gemm_M8192_ws": 521940633,
-    "gemm_M512": 55865418, "gemm_M256": 36992551, "gemm_M256_ws": 70756257, "gemm_M32": 21359785, "gemm_M64": 23724772, "gemm_M128": 28461914,
-    "ffn": 127436248,
+    "gemm_8192": 1300865526, "gemm_8192_ws": 1953975004, "gemm_M8192": 354714344, "gemm_M8192_ws": 521480385,
+    "gemm_M512": 55775304, "gemm_M256": 36883121, "gemm_M256_ws": 70515380, "gemm_M32": 21361191, "gemm_M64": 23731315, "gemm_M128": 28477671,
+    "ffn": 134321304,
 }
 
 
 # where the `traffic` figures come from: counter summaries under profiles/, taken with the library built at this commit
 TRAFFIC_SOURCE = {"streaming": "profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt",
                   "gemm": "profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt",
-                  "library_commit": "9ac7893"}  # the counters were read on the library built from this commit
+                  "library_commit": "6da711b"}  # the counters were read on the library built from this commit
 
 
 def parse():
