@@ -1,7 +1,7 @@
 // Kernel selection for Y = epilogue(X * dequant(W) + bias) with Bfp8_b weights: up to four tile rows ->
 // weight streaming kernel, macro-tile aligned shapes -> the MFMA kernel of gemm_bfp8b_kernel.hpp in
-// one of two tile shapes, a row count that is not a multiple of 128 -> both (rows split), everything
-// else (N or K that do not suit the tiles) -> the bounds-checked general kernel.
+// one of its tile shapes and forms, a row count that is not a multiple of 128 -> both (rows split), N an odd
+// number of tiles -> both (columns split), everything else -> the bounds-checked general kernel.
 #include <cstdlib>
 
 #include "gemm_bfp8b_kernel.hpp"
@@ -25,7 +25,7 @@ hipError_t launch_gemm_bfp8b_skinny(uint32_t M, uint32_t N, uint32_t K, uint32_t
 hipError_t launch_gemm_bfp8b_column_rest(uint32_t M, uint32_t N, uint32_t K, uint32_t ldn, const void *x, const void *w, const void *bias,
                                          int epilogue, void *y, uint8_t y_fmt, hipStream_t stream);
 
-static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x 128), 3 (256 x 256 where it fits), all on two stages; 0 / unset: automatic
+static int force_tile()  // tuning aid: TTBFP_GEMM_TILE = 1 (128 x 64), 2 (128 x 128), 3 (256 x 256), 5 (384 x 128), all on two stages, 6 (192 x 64, two pipelines), each where it fits; 0 / unset: automatic
 {
     static const int force = [] { const char *v = getenv("TTBFP_GEMM_TILE"); return v ? atoi(v) : 0; }();
     return force;
