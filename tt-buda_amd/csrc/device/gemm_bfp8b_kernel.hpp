@@ -538,12 +538,19 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     constexpr uint32_t RAW_PITCH = 2 * RUN_BYTES + (WI * 64 - CPW) * 16;
     static_assert(RAW_CHUNKS % S::NW == 0 && RAW_PITCH % 16 == 0, "raw area: whole pieces per wavefront");
     constexpr uint32_t RAW_BASE = A_RING + 2 * S::B_BYTES;
+    static_assert(RING == 0 || (PW == 4 && KH == 4), "the permutation of the raw rows is written for patches of four rows of one dword");
     uint32_t raw_off[WI];  // offset of this lane's piece from the first tile of the slab (pieces past the end: the last one again)
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
         const uint32_t c = wave * CPW + i * 64 + lane, cc = c < RAW_CHUNKS ? c : RAW_CHUNKS - 1;
         const uint32_t run = cc / (RUN_BYTES / 16), within = cc % (RUN_BYTES / 16);
-        raw_off[i] = run * tiles_n * kW8Tile + within * 16;
+        // inside a tile's data section the 16-byte face rows are permuted (row c lands at c ^ key, key = (face & 1) + 2 (tile
+        // column & 1)): the patch reads of a half-wavefront - one row of two faces of two tiles, both halves of a k chunk -
+        // then fall on 32 different banks instead of 8
+        const uint32_t tile = within / (kW8Tile / 16), piece = within % (kW8Tile / 16);
+        const uint32_t row = piece - kExpSection / 16;  // of the data section, if piece is past the exponents
+        const uint32_t src = piece < kExpSection / 16 ? piece : kExpSection / 16 + (row ^ (((row >> 4) & 1u) | ((tile & 1u) << 1)));
+        raw_off[i] = run * tiles_n * kW8Tile + (tile * (kW8Tile / 16) + src) * 16;
     }
     const uint64_t raw_wave = uniform64((uint64_t)(uintptr_t)Wp + (uint64_t)(n0 / kTile) * kW8Tile + (uint64_t)split * nslabs * w_slab_bytes);
     auto load_x_ring = [&](uint32_t slab, uint32_t slot, auto ic) {
@@ -556,6 +563,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
     };
     // this thread's patch out of a raw area into register set 0: the same units as fetch_w
     const uint32_t raw_patch = (w_kc >> 2) * RUN_BYTES + (w_n / kTile) * kW8Tile;
+    const uint32_t raw_key = ((w_face & 1u) | (((w_n / kTile) & 1u) << 1)) << 4;  // the row permutation above, as a byte offset
     auto fetch_w_ring = [&](uint32_t slot, auto uc) {
         constexpr int U = decltype(uc)::value;
         const uint8_t *t = lds + RAW_BASE + slot * RAW_PITCH + raw_patch;
@@ -568,7 +576,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
             wp[0].d[U - 1][0] = v.x;
             wp[0].d[U - 1][PW / 4 - 1] = v.y;
         } else {
-            wp[0].d[U - 1][0] = *(const uint32_t *)(t + kExpSection + w_in_tile + (U - 1) * 16);
+            wp[0].d[U - 1][0] = *(const uint32_t *)(t + kExpSection + w_in_tile + (raw_key ^ ((U - 1) * 16)));
         }
     };
 
@@ -966,6 +974,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         }
     });
     };
+    if constexpr ((TTBFP_ABLATE & 64) == 0)
     switch (epilogue & kEpilogueMask) {  // uniform
         case 1: finish_blocks(integral_constant<int, 1>{}); break;
         case 2: finish_blocks(integral_constant<int, 2>{}); break;
@@ -980,6 +989,7 @@ __global__ __launch_bounds__(S::NT * GROUPS) void gemm_bfp8b_kernel(uint32_t M, 
         const uint8_t *from = image + row * PITCH + piece * 16;
         uint8_t *to = (uint8_t *)Y + ((uint64_t)(m0 + row) * ldn + n0) * 2 + piece * 16;
         const uint64_t step = (uint64_t)RPP * ldn * 2;
+        if constexpr ((TTBFP_ABLATE & 32) == 0)
         static_for<BM / RPP>([&](auto pc) {
             constexpr int PASS = decltype(pc)::value;
             *(uint4 *)(to + PASS * step) = *(const uint4 *)(from + PASS * RPP * PITCH);
