@@ -29,20 +29,20 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # factor 1.0).  Summary: profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES = {
     # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) x 1024 per launch; the two factors come from the 1 GiB copy in the same runs
-    "tilize_pack": 1644306288,      # 1,644,167,168 algorithmic
-    "unpack_untilize": 1644385769,
+    "tilize_pack": 1644312540,      # 1,644,167,168 algorithmic
+    "unpack_untilize": 1644395026,
     # GEMM kernels, same method: profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt (the forms with a workspace include
     # their first pass / their reduction; the FFN figure is the sum of its two matmuls)
-    "gemm_8192": 1300865526, "gemm_8192_ws": 1953975004, "gemm_M8192": 354714344, "gemm_M8192_ws": 521480385,
-    "gemm_M512": 55775304, "gemm_M256": 36883121, "gemm_M256_ws": 70515380, "gemm_M32": 21361191, "gemm_M64": 23731315, "gemm_M128": 28477671,
-    "ffn": 134321304,
+    "gemm_8192": 1300509562, "gemm_8192_ws": 1953965422, "gemm_M8192": 354743328, "gemm_M8192_ws": 521483661,
+    "gemm_M512": 55775315, "gemm_M256": 36911899, "gemm_M256_ws": 70515940, "gemm_M32": 21361116, "gemm_M64": 23731333, "gemm_M128": 28477861,
+    "ffn": 134321617,
 }
 
 
 # where the `traffic` figures come from: counter summaries under profiles/, taken with the library built at this commit
 TRAFFIC_SOURCE = {"streaming": "profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt",
                   "gemm": "profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt",
-                  "library_commit": "6da711b"}  # the counters were read on the library built from this commit
+                  "library_commit": "e026406"}  # the counters were read on the library built from this commit
 
 
 def parse():
