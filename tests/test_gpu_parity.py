@@ -643,7 +643,8 @@ def test_gemm_with_a_workspace_is_bit_identical(shape, out_dtype):
 
 
 @pytest.mark.parametrize("shape", [(256, 4096, 4096), (256, 1024, 4096), (1024, 1024, 4096), (512, 1024, 4096), (384, 1024, 8192),
-                                   (256, 512, 2048), (256, 512, 2560)])  # the last two: runs of four and of five (an odd number of) slabs
+                                   (256, 512, 2048), (256, 512, 2560),  # these two: runs of four and of five (an odd number of) slabs
+                                   (128, 1024, 4096), (128, 2048, 8192)])  # one tile row: instead of the weight-streaming kernel
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 def test_gemm_split_over_k_with_a_workspace(shape, out_dtype):
     """Shapes whose 128 x 128 tiles leave CUs idle: with a workspace K is cut into runs whose fp32 partial tiles are added

@@ -83,12 +83,14 @@ hipError_t launch_reduce(uint32_t splits, uint64_t quads, uint32_t N, const floa
 // four runs 18.1 / 21.2 (not taken).  The cut with the shortest prediction wins if it saves 3 us or more.
 static uint32_t splitk_factor(uint32_t M, uint32_t N, uint32_t K)
 {
-    if (!gemm_fits<SmallShape>(M, N, K) || K % 64 || M < 256) return 0;  // up to 255 rows go to the weight-streaming kernel
+    if (!gemm_fits<SmallShape>(M, N, K) || K % 64) return 0;  // fewer than 128 rows, and 160 to 224, go to the weight-streaming kernel
     const uint64_t tiles = (uint64_t)(M / 128) * (N / 128);
     if (tiles > 256) return 0;
     const uint32_t slabs = K / BK;
     double fused;
-    if (2 * tiles <= 256)
+    if (M == 128)  // the weight-streaming kernel on four row tiles: every workgroup pulls all of X through its L2 (N = K = 4096: 20 us)
+        fused = 4.3 + 16.0 * ((double)K / 4096.0) * (double)((N + 4095) / 4096);
+    else if (2 * tiles <= 256)
         fused = K % 128 == 0 ? 5.5 + (slabs / 2) * (0.80 + 0.17 * (double)(2 * tiles) / 256.0) : 5.5 + slabs * 0.53;
     else
         fused = K % 128 == 0 ? 5.5 + (slabs / 2) * 1.25 : 5.5 + slabs * 0.735;
