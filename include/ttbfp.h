@@ -233,10 +233,10 @@ int32_t ttbfp_gemm_bfp8b_bf16(uint32_t M, uint32_t N, uint32_t K, const void *x_
 
 /* The same GEMM for callers that can lend scratch memory; ttbfp_gemm_bfp8b_workspace_bytes(M, N, K) says how
  * much a shape can use (0: none).  Two shapes of problem gain from it:
- *  - many rows of X (M >= 3072 or 4096 depending on the tile, macro-tile aligned): W is converted to bf16 once
+ *  - many rows of X (M >= 4096 or 6144 depending on the tile, macro-tile aligned, K a multiple of 64): W is converted to bf16 once
  *    into a panel of 2 K N bytes in the workspace instead of in every workgroup, and the MFMA kernel runs on the
  *    panel; the result is bit-identical to ttbfp_gemm_bfp8b_bf16;
- *  - few macro tiles (256 <= M, fewer than 256 tiles of 128 x 128): K is cut into s <= 8 runs, each (tile, run)
+ *  - few macro tiles (M = 128 or 256 <= M, at most 256 tiles of 128 x 128, K a multiple of 64): K is cut into s <= 8 runs, each (tile, run)
  *    workgroup writes an fp32 partial tile into the workspace (s M N 4 bytes) and a second kernel adds the
  *    partials in a fixed order, then applies bias and epilogue.  Deterministic; the sum is grouped differently
  *    from ttbfp_gemm_bfp8b_bf16's, so the two agree to fp32 rounding (about 1e-7 relative), not bit for bit.
