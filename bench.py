@@ -29,20 +29,20 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # factor 1.0).  Summary: profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES = {
     # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) x 1024 per launch; the two factors come from the 1 GiB copy in the same runs
-    "tilize_pack": 1644312540,      # 1,644,167,168 algorithmic
-    "unpack_untilize": 1644395026,
+    "tilize_pack": 1644306558,      # 1,644,167,168 algorithmic
+    "unpack_untilize": 1644428290,
     # GEMM kernels, same method: profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt (the forms with a workspace include
     # their first pass / their reduction; the FFN figure is the sum of its two matmuls)
-    "gemm_8192": 1300509562, "gemm_8192_ws": 1953965422, "gemm_M8192": 354743328, "gemm_M8192_ws": 521483661,
-    "gemm_M512": 55775315, "gemm_M256": 36911899, "gemm_M256_ws": 70515940, "gemm_M32": 21361116, "gemm_M64": 23731333, "gemm_M128": 28477861,
-    "ffn": 134321617,
+    "gemm_8192": 1287420995, "gemm_8192_ws": 1954009668, "gemm_M8192": 354720605, "gemm_M8192_ws": 521480554,
+    "gemm_M512": 55775136, "gemm_M256": 36911741, "gemm_M256_ws": 70524592, "gemm_M32": 21361155, "gemm_M64": 23731588, "gemm_M128": 28477299,
+    "ffn": 134321260,
 }
 
 
 # where the `traffic` figures come from: counter summaries under profiles/, taken with the library built at this commit
 TRAFFIC_SOURCE = {"streaming": "profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt",
                   "gemm": "profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt",
-                  "library_commit": "e026406"}  # the counters were read on the library built from this commit
+                  "library_commit": "49c267c"}  # the counters were read on the library built from this commit
 
 
 def parse():
