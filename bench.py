@@ -42,7 +42,7 @@ MEASURED_TRAFFIC_BYTES = {
 # where the `traffic` figures come from: counter summaries under profiles/, taken with the library built at this commit
 TRAFFIC_SOURCE = {"streaming": "profiles/streaming_bf16_8x8192x8192_hbm_traffic.txt",
                   "gemm": "profiles/gemm_bfp8b_bench_shapes_hbm_traffic.txt",
-                  "library_commit": "3ab9cde"}  # the counters were read on the library built from this commit
+                  "library_commit": "260d22f"}  # the counters were read on the library built from this commit
 
 
 def parse():
